@@ -11,6 +11,16 @@
 // n_tiles * H * n_splits * (dh + 2) must not exceed it.
 #define DN_DECODE_STATIC_SCRATCH_FLOATS (256 * 1024)
 
+// What a layer may add to the scores of any of the kernels below.  chunk > 0: the row at position p reads only keys from
+// p / chunk * chunk on; bias: 32-bit [H, span], bias[h][p - key] is added to the scaled score (distances from span on take
+// the last entry), or null; sink: a key with score 0 and no value that every row sees.
+struct ScoreExtras {
+  int chunk;
+  const float* bias;
+  int span;
+  int sink;
+};
+
 extern "C" {
 
 // All kernels: q [T, ldq], out [T, ldo] (ldo == 0: packed rows), k_pool [n_pages, Hkv, page_size, dh],
@@ -21,6 +31,17 @@ int dn_attention(const void* q, int ldq, void* out, int ldo, const void* k_pool,
                  const int32_t* block_tables, int max_blocks, const int32_t* tile_seq, const int32_t* tile_row0,
                  const int32_t* tile_nrows, const int32_t* tile_pos0, int n_tiles, int H, int Hkv, int dh,
                  int page_size, float scale, int window, int dtype, hipStream_t stream);
+
+// dn_attention with chunks, a bias by distance and a sink (ScoreExtras)
+int dn_attention_extras(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
+                        const int32_t* block_tables, int max_blocks, const int32_t* tile_seq, const int32_t* tile_row0,
+                        const int32_t* tile_nrows, const int32_t* tile_pos0, int n_tiles, int H, int Hkv, int dh,
+                        int page_size, float scale, int window, int chunk, const float* bias, int span, int sink, int dtype,
+                        hipStream_t stream);
+int dn_attention_rows_extras(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
+                             const int32_t* block_tables, int max_blocks, const int32_t* tile_seq, const int32_t* tile_pos0,
+                             int n_tiles, float* part, int max_context, int H, int Hkv, int dh, int page_size, float scale,
+                             int window, int chunk, const float* bias, int span, int sink, int dtype, hipStream_t stream);
 
 // the same kernels' arithmetic for a step of single rows (tile s = request s = row s), every tile of keys a
 // workgroup of its own; part: n_tiles * H * ceil(max_context / dn_attention_rows_tile(dh)) * (dh + 2) floats

@@ -8,6 +8,11 @@
 // length and the softmax is the running ("online") one in 32-bit, so a row's result does not
 // depend on where its portion was cut or on what else is in the batch.
 //
+// What a layer may add to this (ScoreExtras): chunks (a row reads only the keys of its own run of `chunk` positions, runs
+// counted from the request's position 0), a bias by distance (bias[h][pos - key] is added to the scaled score; distances
+// from `span` on take the last entry) and a sink (a key that every row sees, with score 0 and no value: one more
+// summand, exp(0), under the softmax).
+//
 // The key pool is [n_pages, Hkv, page_size, dh], the value pool [n_pages, Hkv, dh, page_size];
 // query head h reads key head h / (H / Hkv).
 #include "common.h"
@@ -16,6 +21,13 @@
 #include <math.h>
 
 #include <mutex>
+
+// the first key that the row at `pos` reads
+__device__ __forceinline__ int first_key(int pos, int window, int chunk) {
+  int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  if (chunk > 0) lo = max(lo, pos / chunk * chunk);
+  return lo;
+}
 
 namespace plain {
 constexpr int BQ = 16;
@@ -59,7 +71,8 @@ __device__ __forceinline__ float dim_sum(const float* ps, const float* vs, int d
 
 // the scores of one row against the tile in Ks: p[j] to Ps (this row's BK entries), -> m_T, l_T
 __device__ __forceinline__ void tile_scores(const float* qr, const float* Ks, float* ps, int g, int nc, int dh, int kt,
-                                            int lo, int pos, bool row_ok, float scale, float& m_t, float& l_t) {
+                                            int lo, int pos, bool row_ok, float scale, const float* bias, int span, float& m_t,
+                                            float& l_t) {
   const float NEG_INF = -INFINITY;
   float s[4];
   float tmax = NEG_INF;
@@ -71,7 +84,7 @@ __device__ __forceinline__ void tile_scores(const float* qr, const float* Ks, fl
       const int key = kt + j;
       const float dot = key_dot(qr, Ks + j * (dh + 1), dh);
       const bool ok = row_ok && key >= lo && key <= pos;
-      s[c] = ok ? dot * scale : NEG_INF;
+      s[c] = ok ? (bias ? fmaf(dot, scale, bias[min(pos - key, span - 1)]) : dot * scale) : NEG_INF;
       tmax = fmaxf(tmax, s[c]);
     }
   }
@@ -187,7 +200,7 @@ __global__ __launch_bounds__(THREADS) void attention_kernel(
     const T* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_row0,
     const int32_t* __restrict__ tile_nrows, const int32_t* __restrict__ tile_pos0, int H, int Hkv, int dh,
-    int page_size, int BK, float scale, int window) {
+    int page_size, int BK, float scale, int window, ScoreExtras ex) {
   // A head size that is no multiple of 16 lies in LDS padded to the next one (dhp): the dims beyond dh are
   // zeros in the queries and the keys, add nothing to a score (a fused multiply-add of zeros leaves a sum as
   // it is), and are not stored; the real dims keep their order of summation.
@@ -219,9 +232,10 @@ __global__ __launch_bounds__(THREADS) void attention_kernel(
   }
   const bool row_ok = qi < nrows;
   const int my_pos = pos0 + qi;
-  const int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
+  const int my_lo = first_key(my_pos, window, ex.chunk);
   const int last_pos = pos0 + nrows - 1;
-  const int first_lo = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int first_lo = first_key(pos0, window, ex.chunk);
+  const float* bias = ex.bias ? ex.bias + static_cast<size_t>(h) * ex.span : nullptr;
   const int nd = dhp / 16, nc = BK / 16;
 
   float m = NEG_INF, l = 0.f;
@@ -233,7 +247,7 @@ __global__ __launch_bounds__(THREADS) void attention_kernel(
     __syncthreads();
     load_tile(Ks, Vs, Kb, Vb, k_pool, v_pool, bt, kt, last_pos, BK, dh, page_size, Hkv, hk, dhp + 1);
     float m_t, l_t, a_t[16];
-    tile_scores(Qs + qi * dhp, Ks, Ps + qi * BK, g, nc, dhp, kt, my_lo, my_pos, row_ok, scale, m_t, l_t);
+    tile_scores(Qs + qi * dhp, Ks, Ps + qi * BK, g, nc, dhp, kt, my_lo, my_pos, row_ok, scale, bias, ex.span, m_t, l_t);
     __syncthreads();
     if (m_t > NEG_INF) {                // the same for the 16 threads of a row
       tile_values(Ps + qi * BK, Vs, g, nd, dhp, BK, a_t);
@@ -241,7 +255,7 @@ __global__ __launch_bounds__(THREADS) void attention_kernel(
     }
   }
   if (row_ok) {
-    float inv = 1.0f / l;
+    float inv = 1.0f / (ex.sink ? l + expf(-m) : l);
     T* o = out + static_cast<size_t>(row0 + qi) * ldo + h * dh;
 #pragma unroll
     for (int i = 0; i < 16; ++i)
@@ -258,7 +272,7 @@ __global__ __launch_bounds__(THREADS) void row_tiles_kernel(
     const T* __restrict__ q, int ldq, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ tile_seq,
     const int32_t* __restrict__ tile_pos0, float* __restrict__ part, int n_key_tiles, int H, int Hkv, int dh,
-    int page_size, int BK, float scale, int window) {
+    int page_size, int BK, float scale, int window, ScoreExtras ex) {
   extern __shared__ float smem[];
   float* Qs = smem;                    // [dh]
   float* Ks = Qs + dh;                 // [BK][dh + 1]
@@ -270,7 +284,8 @@ __global__ __launch_bounds__(THREADS) void row_tiles_kernel(
   const int seq = tile_seq[tile];
   if (seq < 0) return;
   const int pos = tile_pos0[tile];
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = first_key(pos, window, ex.chunk);
+  const float* bias = ex.bias ? ex.bias + static_cast<size_t>(h) * ex.span : nullptr;
   const int kt = ktile * BK;
   const int t = threadIdx.x, g = t % 16;
   float* mine = part + ((static_cast<size_t>(tile) * H + h) * n_key_tiles + ktile) * (dh + 2);
@@ -291,7 +306,7 @@ __global__ __launch_bounds__(THREADS) void row_tiles_kernel(
     if (t < BK) {
       const int key = kt + t;
       const float dot = key_dot(Qs, Ks + t * (dh + 1), dh);
-      s = (key >= lo && key <= pos) ? dot * scale : NEG_INF;
+      s = (key >= lo && key <= pos) ? (bias ? fmaf(dot, scale, bias[min(pos - key, ex.span - 1)]) : dot * scale) : NEG_INF;
     }
     const float tmax = wave_max(s);
     if (t < BK) Ps[t] = s > NEG_INF ? expf(s - tmax) : 0.f;
@@ -335,7 +350,7 @@ __global__ __launch_bounds__(64) void row_tile64_kernel(
     const T* __restrict__ q, int ldq, const T* __restrict__ k_pool, const T* __restrict__ v_pool,
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ tile_seq,
     const int32_t* __restrict__ tile_pos0, float* __restrict__ part, int n_key_tiles, int H, int Hkv, int page_size,
-    float scale, int window) {
+    float scale, int window, ScoreExtras ex) {
   constexpr int DH = 64, BK = 64, LD = DH + 4, QUADS = BK / 4;
   __shared__ __attribute__((aligned(16))) float Ks[BK * LD];
   __shared__ __attribute__((aligned(16))) float Qs[DH];
@@ -344,7 +359,8 @@ __global__ __launch_bounds__(64) void row_tile64_kernel(
   const int seq = tile_seq[tile];
   if (seq < 0) return;
   const int pos = tile_pos0[tile];
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = first_key(pos, window, ex.chunk);
+  const float* bias = ex.bias ? ex.bias + static_cast<size_t>(h) * ex.span : nullptr;
   const int kt = ktile * BK;
   const int lane = threadIdx.x;
   float* mine = part + ((static_cast<size_t>(tile) * H + h) * n_key_tiles + ktile) * (DH + 2);
@@ -393,7 +409,7 @@ __global__ __launch_bounds__(64) void row_tile64_kernel(
     dot = fmaf(a.w, b.w, dot);
   }
   const int key = kt + lane;
-  const float sc = (key >= lo && key <= pos) ? dot * scale : NEG_INF;
+  const float sc = (key >= lo && key <= pos) ? (bias ? fmaf(dot, scale, bias[min(pos - key, ex.span - 1)]) : dot * scale) : NEG_INF;
   const float tmax = wave_max(sc);
   Ps[lane] = sc > NEG_INF ? expf(sc - tmax) : 0.f;
   __syncthreads();
@@ -422,7 +438,7 @@ __global__ __launch_bounds__(64) void row_tile64_kernel(
 
 template <typename T>
 __global__ void row_join_kernel(const float* __restrict__ part, T* __restrict__ out, int ldo,
-                                const int32_t* __restrict__ tile_seq, int n_key_tiles, int H, int dh) {
+                                const int32_t* __restrict__ tile_seq, int n_key_tiles, int H, int dh, int sink) {
   const int tile = blockIdx.x, h = blockIdx.y;
   if (tile_seq[tile] < 0) return;
   const int g = threadIdx.x;           // 16 threads, the dims g + 16 i each, as in the kernels above
@@ -452,7 +468,7 @@ __global__ void row_join_kernel(const float* __restrict__ part, T* __restrict__ 
       join_tile(m, l, acc, m_t[u], l_t[u], a_t, nd);
     }
   }
-  const float inv = 1.0f / l;
+  const float inv = 1.0f / (sink ? l + expf(-m) : l);
   T* o = out + static_cast<size_t>(tile) * ldo + h * dh;
 #pragma unroll
   for (int i = 0; i < 16; ++i)
@@ -468,7 +484,18 @@ extern "C" int dn_attention(const void* q, int ldq, void* out, int ldo, const vo
                             const int32_t* tile_row0, const int32_t* tile_nrows, const int32_t* tile_pos0,
                             int n_tiles, int H, int Hkv, int dh, int page_size, float scale, int window, int dtype,
                             hipStream_t stream) {
+  return dn_attention_extras(q, ldq, out, ldo, k_pool, v_pool, block_tables, max_blocks, tile_seq, tile_row0, tile_nrows, tile_pos0,
+                             n_tiles, H, Hkv, dh, page_size, scale, window, 0, nullptr, 0, 0, dtype, stream);
+}
+
+extern "C" int dn_attention_extras(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
+                                   const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,
+                                   const int32_t* tile_row0, const int32_t* tile_nrows, const int32_t* tile_pos0,
+                                   int n_tiles, int H, int Hkv, int dh, int page_size, float scale, int window, int chunk,
+                                   const float* bias, int span, int sink, int dtype, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
+  if (chunk < 0 || (bias && span < 1)) return DN_ERR_SHAPE;
+  const ScoreExtras ex{chunk, bias, span, sink};
   // (any head size up to 256: one that is no multiple of 16 is padded to the next inside the kernel)
   if (dh < 1 || dh > 256 || Hkv < 1 || H % Hkv != 0 || page_size < 1 || max_blocks < 1) return DN_ERR_SHAPE;
   const int dhp = (dh + 15) / 16 * 16;
@@ -480,12 +507,12 @@ extern "C" int dn_attention(const void* q, int ldq, void* out, int ldo, const vo
     hipLaunchKernelGGL(plain::attention_kernel<float>, grid, block, lds, stream, static_cast<const float*>(q), ldq,
                        static_cast<float*>(out), ldo, static_cast<const float*>(k_pool),
                        static_cast<const float*>(v_pool), block_tables, max_blocks, tile_seq, tile_row0, tile_nrows,
-                       tile_pos0, H, Hkv, dh, page_size, BK, scale, window);
+                       tile_pos0, H, Hkv, dh, page_size, BK, scale, window, ex);
   else if (dtype == DN_BF16)
     hipLaunchKernelGGL(plain::attention_kernel<bf16_t>, grid, block, lds, stream, static_cast<const bf16_t*>(q),
                        ldq, static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(k_pool),
                        static_cast<const bf16_t*>(v_pool), block_tables, max_blocks, tile_seq, tile_row0,
-                       tile_nrows, tile_pos0, H, Hkv, dh, page_size, BK, scale, window);
+                       tile_nrows, tile_pos0, H, Hkv, dh, page_size, BK, scale, window, ex);
   else
     return DN_ERR_DTYPE;
   return dn_launch_status();
@@ -500,7 +527,18 @@ extern "C" int dn_attention_rows(const void* q, int ldq, void* out, int ldo, con
                                  const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,
                                  const int32_t* tile_pos0, int n_tiles, float* part, int max_context, int H, int Hkv,
                                  int dh, int page_size, float scale, int window, int dtype, hipStream_t stream) {
+  return dn_attention_rows_extras(q, ldq, out, ldo, k_pool, v_pool, block_tables, max_blocks, tile_seq, tile_pos0, n_tiles, part,
+                                  max_context, H, Hkv, dh, page_size, scale, window, 0, nullptr, 0, 0, dtype, stream);
+}
+
+extern "C" int dn_attention_rows_extras(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
+                                        const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,
+                                        const int32_t* tile_pos0, int n_tiles, float* part, int max_context, int H, int Hkv,
+                                        int dh, int page_size, float scale, int window, int chunk, const float* bias, int span,
+                                        int sink, int dtype, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
+  if (chunk < 0 || (bias && span < 1)) return DN_ERR_SHAPE;
+  const ScoreExtras ex{chunk, bias, span, sink};
   if (dh < 16 || dh > 256 || dh % 16 != 0 || Hkv < 1 || H % Hkv != 0 || page_size < 1 || max_blocks < 1 ||
       max_context < 1 || !part || n_tiles > 65535 || H > 65535)
     return DN_ERR_SHAPE;
@@ -514,13 +552,13 @@ extern "C" int dn_attention_rows(const void* q, int ldq, void* out, int ldo, con
   if (wave_tiles)                                                                                                    \
     hipLaunchKernelGGL(plain::row_tile64_kernel<T>, grid, dim3(64), 0, stream, static_cast<const T*>(q), ldq,        \
                        static_cast<const T*>(k_pool), static_cast<const T*>(v_pool), block_tables, max_blocks,       \
-                       tile_seq, tile_pos0, part, n_key_tiles, H, Hkv, page_size, scale, window);                    \
+                       tile_seq, tile_pos0, part, n_key_tiles, H, Hkv, page_size, scale, window, ex);                \
   else                                                                                                               \
     hipLaunchKernelGGL(plain::row_tiles_kernel<T>, grid, block, lds, stream, static_cast<const T*>(q), ldq,          \
                        static_cast<const T*>(k_pool), static_cast<const T*>(v_pool), block_tables, max_blocks,       \
-                       tile_seq, tile_pos0, part, n_key_tiles, H, Hkv, dh, page_size, BK, scale, window);            \
+                       tile_seq, tile_pos0, part, n_key_tiles, H, Hkv, dh, page_size, BK, scale, window, ex);        \
   hipLaunchKernelGGL(plain::row_join_kernel<T>, dim3(n_tiles, H), dim3(16), 0, stream, part, static_cast<T*>(out), ldo, \
-                     tile_seq, n_key_tiles, H, dh)
+                     tile_seq, n_key_tiles, H, dh, sink)
   if (dtype == DN_F32) {
     DN_ROWS(float);
   } else if (dtype == DN_BF16) {

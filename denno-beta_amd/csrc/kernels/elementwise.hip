@@ -130,6 +130,46 @@ extern "C" int dn_embed(const int32_t* tokens, const int32_t* positions, const v
 }
 
 // ---------------------------------------------------------------------------------------
+// Rows of a table that the pair (token before, token) picks: out[t] = (prev * mul_prev + token * mul_cur) mod buckets, in
+// 64-bit; a request's first token (position 0) has no token before it and takes row `buckets`, the table's last.  The
+// token before a step's first row of a request is the request's state last[slot]; the thread of that row also leaves the
+// request's last token of this step there (if `write`), after it has read.  Padding (slot < 0) reads and writes no state.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void pair_rows_kernel(const int32_t* __restrict__ tokens, const int32_t* __restrict__ positions,
+                                                        const int32_t* __restrict__ row_start, const int32_t* __restrict__ slots, int S,
+                                                        int32_t* __restrict__ last, long long last_stride, long long mul_prev,
+                                                        long long mul_cur, int buckets, int write, int32_t* __restrict__ out, int T) {
+  const int t = blockIdx.x * 256 + threadIdx.x;
+  if (t >= T) return;
+  int lo = 0, hi = S - 1;
+  while (lo < hi) {
+    const int mid = (lo + hi + 1) >> 1;
+    if (row_start[mid] <= t) lo = mid; else hi = mid - 1;
+  }
+  const int s = lo, slot = slots[s];
+  const bool first = t == row_start[s], live = slot >= 0 && t < row_start[S];
+  int row = buckets;
+  if (positions[t] > 0) {
+    long long prev = -1;
+    if (!first) prev = tokens[t - 1];
+    else if (live) prev = last[slot * last_stride];
+    if (prev >= 0) row = static_cast<int>((prev * mul_prev + static_cast<long long>(tokens[t]) * mul_cur) % buckets);
+  }
+  out[t] = row;
+  if (first && live && write) last[slot * last_stride] = tokens[row_start[s + 1] - 1];
+}
+
+extern "C" int dn_pair_rows(const int32_t* tokens, const int32_t* positions, const int32_t* row_start, const int32_t* slots, int S,
+                            int32_t* last, long long last_stride, long long mul_prev, long long mul_cur, int buckets, int write,
+                            int32_t* out, int T, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (S < 1 || buckets < 1 || mul_prev < 0 || mul_cur < 0) return DN_ERR_SHAPE;
+  hipLaunchKernelGGL(pair_rows_kernel, dim3((T + 255) / 256), dim3(256), 0, stream, tokens, positions, row_start, slots, S, last,
+                     last_stride, mul_prev, mul_cur, buckets, write, out, T);
+  return dn_launch_status();
+}
+
+// ---------------------------------------------------------------------------------------
 // LayerNorm of selected rows: mean, biased variance of (x - mean), then affine
 // (crates/denno-engine/src/tensor.rs:1101-1112).  One wave per row; the row is read three
 // times (it stays in cache), so any width works.  rows == null: row r of the output is

@@ -116,8 +116,9 @@ __global__ __launch_bounds__(256) void concat_kernel(const float* a, size_t lda,
 // ---- short causal convolution over time ----------------------------------------------------------------------
 // out[t, c] = act((identity ? h[t, c] : 0) + sum_j w[c, j] * h[t - taps + 1 + j, c]); rows before the step's first row of a
 // request come from its history [slot][taps - 1][width] (oldest first; zero for a new request).  h and out are rows
-// ldh and ldo numbers apart (the channels may be the first columns of wider rows); act: none or silu.
-__global__ __launch_bounds__(256) void conv_rows_kernel(const float* h, size_t ldh, const float* w, const float* hist, const int* row_start,
+// ldh and ldo numbers apart (the channels may be the first columns of wider rows); act: none or silu; bias: a number per
+// channel that the sum starts from, or none.
+__global__ __launch_bounds__(256) void conv_rows_kernel(const float* h, size_t ldh, const float* w, const float* bias, const float* hist, const int* row_start,
                                                         const int* slots, int S, int width, int taps, int identity, int silu, void* out,
                                                         int out_dt, size_t ldo, size_t hist_stride) {
   const int t = blockIdx.x;
@@ -130,7 +131,7 @@ __global__ __launch_bounds__(256) void conv_rows_kernel(const float* h, size_t l
   const int i = t - row_start[s];
   const float* past = hist + static_cast<size_t>(slot) * hist_stride;
   for (int c = threadIdx.x; c < width; c += 256) {
-    float acc = identity ? h[static_cast<size_t>(t) * ldh + c] : 0.f;
+    float acc = (identity ? h[static_cast<size_t>(t) * ldh + c] : 0.f) + (bias ? bias[c] : 0.f);
     for (int j = 0; j < taps; ++j) {
       const int src = i - taps + 1 + j;
       const float v = src >= 0 ? h[static_cast<size_t>(row_start[s] + src) * ldh + c] : past[static_cast<size_t>(i + j) * width + c];
@@ -350,7 +351,8 @@ __global__ __launch_bounds__(256) void gated_kernel(const void* x, int x_dt, siz
 //   read_after:   S_i <- w_i S_i + a_i v_j ;  o_j = sum_i r_i S_i
 //   delta:        S_i <- w_i S_i ;  e_j = beta (v_j - sum_i a_i S_i) ;  S_i <- S_i + a_i e_j ;  o_j = sum_i r_i S_i
 //   else:         o_j = sum_i r_i (S_i + u_i a_i v_j) ;  S_i <- w_i S_i + a_i v_j
-// w is a number per row, head and key channel, or (w_head) one per head for all rows and channels.  r and k may have
+// w is a number per row, head and key channel, or (w_rows) one per row and head for all the head's channels, or (w_head) one
+// per head for all rows and channels.  r and k may have
 // fewer heads than v: head h reads r and k of head h / (H / G).
 // A column's key channels are shared out among KG lanes that lie side by side (4 lanes for heads of up to 32 key
 // channels, 16 beyond), so a wave has 64 / KG columns and a column's parts are joined inside a row of 16 lanes,
@@ -368,7 +370,7 @@ struct ScanArgs {
   float* state;
   size_t slot_stride;
   const int *row_start, *slots;
-  int H, dk, dv, read_after, key_from_decay, beta_logits;
+  int H, dk, dv, read_after, key_from_decay, beta_logits, w_rows;
   float* out;
   size_t ldo;
 };
@@ -417,7 +419,7 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
         const bool ok = idx < N4 && t < row1 && i < dk;
         r4[it] = ok ? *reinterpret_cast<const f32x4*>(a.r + t * a.ldr + hq * dk + i) : zero;
         k4[it] = (ok && !a.key_from_decay) ? *reinterpret_cast<const f32x4*>(a.k + t * a.ldk + hq * dk + i) : zero;
-        w4[it] = !ok ? one : a.w_head ? one * wh : *reinterpret_cast<const f32x4*>(a.w + t * a.ldw + h * dk + i);
+        w4[it] = !ok ? one : a.w_head ? one * wh : a.w_rows ? one * a.w[t * a.ldw + h] : *reinterpret_cast<const f32x4*>(a.w + t * a.ldw + h * dk + i);
       }
       if constexpr (DELTA) nb[0] = (lane < TB && t0 + lane < row1) ? beta_of(a.beta[(t0 + lane) * a.ldb + h]) : 0.f;
       const int bq = lane / (CW / 4), col = j0 + (lane % (CW / 4)) * 4, t = t0 + bq;
@@ -433,7 +435,7 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
           const bool ok = row && i < dk;
           nr[bq][q] = ok ? a.r[t * a.ldr + hq * dk + i] : 0.f;
           nk[bq][q] = (ok && !a.key_from_decay) ? a.k[t * a.ldk + hq * dk + i] : 0.f;
-          nw[bq][q] = !ok ? 1.f : a.w_head ? wh : a.w[t * a.ldw + h * dk + i];
+          nw[bq][q] = !ok ? 1.f : a.w_head ? wh : a.w_rows ? a.w[t * a.ldw + h] : a.w[t * a.ldw + h * dk + i];
         }
         if constexpr (DELTA) nb[bq] = row ? beta_of(a.beta[t * a.ldb + h]) : 0.f;
         nv[bq] = (row && live) ? a.v[t * a.ldv + h * dv + j] : 0.f;
@@ -537,41 +539,203 @@ __global__ __launch_bounds__(64) void scan_kernel(ScanArgs a) {
 }
 
 // ---- a norm per head, with a gate ----------------------------------------------------------------------------
-// out[t, h, j] = o[t, h, j] / sqrt(mean_j(o^2) + eps) * weight[h * w_stride + j] * act(gate[t, h, j]); a wave a head.
-__global__ __launch_bounds__(64) void head_norm_kernel(const float* o, size_t ld, const float* weight, int w_stride, float eps,
-                                                       const float* gate, size_t ldg, int gate_kind, void* out, int out_dt,
-                                                       size_t ldo, int dv) {
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  const float* src = o + t * ld + static_cast<size_t>(h) * dv;
+// y = o[t, h, j] (+ skip[t, h * dv + j] * skip_scale[(h * dv + j) / skip_dim], a second summand with a number per run of
+// skip_dim columns); gate_first: y *= act(gate) before the norm, else behind it;
+// out[t, h, j] = y / sqrt(mean_j(y^2) + eps) * weight[h * w_stride + j]; a wave a head.
+struct HeadNormArgs {
+  const float* o; size_t ld;
+  const float* weight; int w_stride; float eps;
+  const float* gate; size_t ldg; int gate_kind, gate_first;
+  const float* skip; size_t lds; const float* skip_scale; int skip_dim;
+  void* out; int out_dt; size_t ldo; int dv;
+};
+
+__device__ __forceinline__ float head_norm_in(const HeadNormArgs& a, size_t t, int col) {
+  float y = a.o[t * a.ld + col];
+  if (a.skip) y = fmaf(a.skip[t * a.lds + col], a.skip_scale[col / a.skip_dim], y);
+  if (a.gate && a.gate_first) y *= activation(a.gate_kind, a.gate[t * a.ldg + col], 0.f);
+  return y;
+}
+
+__global__ __launch_bounds__(64) void head_norm_kernel(HeadNormArgs a) {
+  const int h = blockIdx.y, lane = threadIdx.x, dv = a.dv;
+  const size_t t = blockIdx.x;
   float ss = 0.f;
-  for (int j = lane; j < dv; j += 64) ss = fmaf(src[j], src[j], ss);
-  ss = wave_sum(ss);
-  const float inv = 1.0f / sqrtf(ss / static_cast<float>(dv) + eps);
   for (int j = lane; j < dv; j += 64) {
-    float y = src[j] * inv;
-    if (weight) y *= weight[h * w_stride + j];
-    if (gate) y *= activation(gate_kind, gate[t * ldg + static_cast<size_t>(h) * dv + j], 0.f);
-    store_as(out, t * ldo + static_cast<size_t>(h) * dv + j, out_dt, y);
+    const float y = head_norm_in(a, t, h * dv + j);
+    ss = fmaf(y, y, ss);
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(dv) + a.eps);
+  for (int j = lane; j < dv; j += 64) {
+    float y = head_norm_in(a, t, h * dv + j) * inv;
+    if (a.weight) y *= a.weight[h * a.w_stride + j];
+    if (a.gate && !a.gate_first) y *= activation(a.gate_kind, a.gate[t * a.ldg + static_cast<size_t>(h) * dv + j], 0.f);
+    store_as(a.out, t * a.ldo + static_cast<size_t>(h) * dv + j, a.out_dt, y);
   }
 }
 
 // The same for heads of many columns (all heads normed as one vector): a workgroup a head, the sums as in rmsnorm_kernel.
 // Which of the two kernels runs depends on the head's size alone.
-__global__ __launch_bounds__(256) void head_norm_wide_kernel(const float* o, size_t ld, const float* weight, int w_stride, float eps,
-                                                             const float* gate, size_t ldg, int gate_kind, void* out, int out_dt,
-                                                             size_t ldo, int dv) {
+__global__ __launch_bounds__(256) void head_norm_wide_kernel(HeadNormArgs a) {
   __shared__ float sh[4];
-  const int t = blockIdx.x, h = blockIdx.y;
-  const float* src = o + t * ld + static_cast<size_t>(h) * dv;
+  const int h = blockIdx.y, dv = a.dv;
+  const size_t t = blockIdx.x;
   float ss = 0.f;
-  for (int j = threadIdx.x; j < dv; j += 256) ss = fmaf(src[j], src[j], ss);
-  ss = block_sum_256(ss, sh);
-  const float inv = 1.0f / sqrtf(ss / static_cast<float>(dv) + eps);
   for (int j = threadIdx.x; j < dv; j += 256) {
-    float y = src[j] * inv;
-    if (weight) y *= weight[h * w_stride + j];
-    if (gate) y *= activation(gate_kind, gate[t * ldg + static_cast<size_t>(h) * dv + j], 0.f);
-    store_as(out, t * ldo + static_cast<size_t>(h) * dv + j, out_dt, y);
+    const float y = head_norm_in(a, t, h * dv + j);
+    ss = fmaf(y, y, ss);
+  }
+  ss = block_sum_256(ss, sh);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(dv) + a.eps);
+  for (int j = threadIdx.x; j < dv; j += 256) {
+    float y = head_norm_in(a, t, h * dv + j) * inv;
+    if (a.weight) y *= a.weight[h * a.w_stride + j];
+    if (a.gate && !a.gate_first) y *= activation(a.gate_kind, a.gate[t * a.ldg + static_cast<size_t>(h) * dv + j], 0.f);
+    store_as(a.out, t * a.ldo + static_cast<size_t>(h) * dv + j, a.out_dt, y);
+  }
+}
+
+// ---- what a state-space recurrence with one decay per head reads -------------------------------------------------
+// dt = log(1 + e^(z[t, h] + bias[h])); decay[t, h] = exp(-rate[h] * dt); v[t, h, :] = dt * x[t, h, :].  A workgroup a row.
+__global__ __launch_bounds__(256) void step_sizes_kernel(const float* z, size_t ldz, const float* bias, const float* rate, const float* x,
+                                                         size_t ldx, int H, int dv, float* decay, size_t ldd, float* v, size_t ldv) {
+  const size_t t = blockIdx.x;
+  for (int h = threadIdx.x; h < H; h += 256) decay[t * ldd + h] = expf(-rate[h] * softplus_f(z[t * ldz + h] + (bias ? bias[h] : 0.f)));
+  for (int c = threadIdx.x; c < H * dv; c += 256) {
+    const int h = c / dv;
+    v[t * ldv + c] = softplus_f(z[t * ldz + h] + (bias ? bias[h] : 0.f)) * x[t * ldx + c];
+  }
+}
+
+// ---- a recurrence of single numbers whose gates read the token alone ----------------------------------------------
+// z = sigmoid(a[t, c] + bias_a[c]); u = b[t, c] + bias_b[c]; cand = u >= 0 ? u + 1/2 : sigmoid(u); S <- (1 - z) S + z cand;
+// out[t, c] = S * silu(g[t, c]).  A thread owns a channel of a request and walks its rows in order; eight rows' numbers are
+// asked for at a time, the next eight before the current ones are worked on.  A row's result depends on the rows before it
+// alone, in one order.
+__global__ __launch_bounds__(64) void gate_scan_kernel(const float* a, size_t lda, const float* b, size_t ldb, const float* g, size_t ldg,
+                                                       const float* bias_a, const float* bias_b, float* state, size_t slot_stride,
+                                                       const int* row_start, const int* slots, int width, void* out, int out_dt,
+                                                       size_t ldo) {
+  constexpr int TB = 8;
+  const int s = blockIdx.y, c = blockIdx.x * 64 + threadIdx.x;
+  const int slot = slots[s];
+  if (slot < 0 || c >= width) return;
+  const int row0 = row_start[s], row1 = row_start[s + 1];
+  if (row0 >= row1) return;
+  const float ba = bias_a ? bias_a[c] : 0.f, bb = bias_b ? bias_b[c] : 0.f;
+  float* sp = state + static_cast<size_t>(slot) * slot_stride + c;
+  float S = *sp;
+  float na[TB], nb[TB], ng[TB];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      const size_t t = min(t0 + i, row1 - 1);
+      na[i] = a[t * lda + c], nb[i] = b[t * ldb + c], ng[i] = g[t * ldg + c];
+    }
+  };
+  fetch(row0);
+  for (int t0 = row0; t0 < row1; t0 += TB) {
+    float ca[TB], cb[TB], cg[TB];
+#pragma unroll
+    for (int i = 0; i < TB; ++i) ca[i] = na[i], cb[i] = nb[i], cg[i] = ng[i];
+    if (t0 + TB < row1) fetch(t0 + TB);
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      if (t0 + i < row1) {
+        const float z = sigmoid_f(ca[i] + ba), u = cb[i] + bb;
+        const float cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
+        S = fmaf(z, cand - S, S);
+        store_as(out, static_cast<size_t>(t0 + i) * ldo + c, out_dt, S * activation(ACT_SILU, cg[i], 0.f));
+      }
+    }
+  }
+  *sp = S;
+}
+
+// ---- several copies of the stream -----------------------------------------------------------------------------------
+// The stream as n copies [n][rows][width], `plane` numbers apart.
+// read: u = sum_s w_in[s] x_s[row] (s ascending, one fused multiply-add a step; w_in none: the plain sum), then
+// out[r] = u / sqrt(mean(u^2) + eps) * g (g: a number per column; none, with eps < 0: u itself).  One workgroup a row.
+constexpr int STREAMS_MAX = 8;
+
+__global__ __launch_bounds__(256) void streams_read_kernel(const float* xs, size_t plane, int n, const float* w_in, const float* g, float eps,
+                                                           void* out, int out_dt, size_t ldo, const int* rows, int width) {
+  __shared__ float sh[4];
+  const int r = blockIdx.x;
+  const size_t src = static_cast<size_t>(rows ? rows[r] : r) * width;
+  float wi[STREAMS_MAX];
+#pragma unroll
+  for (int s = 0; s < STREAMS_MAX; ++s) wi[s] = s < n ? (w_in ? w_in[s] : 1.0f) : 0.f;
+  const bool normed = eps >= 0.f;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float u = 0.f;
+#pragma unroll
+    for (int s = 0; s < STREAMS_MAX; ++s)
+      if (s < n) u = fmaf(wi[s], xs[s * plane + src + c], u);
+    ss = fmaf(u, u, ss);
+  }
+  float inv = 1.0f;
+  if (normed) {
+    ss = block_sum_256(ss, sh);
+    inv = 1.0f / sqrtf(ss / static_cast<float>(width) + eps);
+  }
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float u = 0.f;
+#pragma unroll
+    for (int s = 0; s < STREAMS_MAX; ++s)
+      if (s < n) u = fmaf(wi[s], xs[s * plane + src + c], u);
+    u *= inv;
+    store_as(out, static_cast<size_t>(r) * ldo + c, out_dt, g ? u * g[c] : u);
+  }
+}
+
+// write: every copy anew from the old ones and a sublayer's result y: x_t <- sum_s mix[s][t] x_s + w_out[t] * y (s ascending).
+// next_in given: the same workgroup then reads the new copies for the next sublayer, as streams_read_kernel does, into `out`.
+__global__ __launch_bounds__(256) void streams_write_kernel(float* xs, size_t plane, int n, const float* mix, const float* w_out, const float* y,
+                                                            size_t ldy, const float* next_in, const float* g, float eps, void* out, int out_dt,
+                                                            size_t ldo, int width) {
+  __shared__ float sh[4];
+  __shared__ float sm[STREAMS_MAX * STREAMS_MAX + 2 * STREAMS_MAX];
+  const size_t row = blockIdx.x;
+  if (threadIdx.x < n * n) sm[threadIdx.x] = mix[threadIdx.x];
+  if (threadIdx.x < n) {
+    sm[STREAMS_MAX * STREAMS_MAX + threadIdx.x] = w_out[threadIdx.x];
+    sm[STREAMS_MAX * STREAMS_MAX + STREAMS_MAX + threadIdx.x] = next_in ? next_in[threadIdx.x] : 0.f;
+  }
+  __syncthreads();
+  const float* wo = sm + STREAMS_MAX * STREAMS_MAX;
+  const float* wn = wo + STREAMS_MAX;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float old[STREAMS_MAX];
+#pragma unroll
+    for (int s = 0; s < STREAMS_MAX; ++s) old[s] = s < n ? xs[s * plane + row * width + c] : 0.f;
+    const float yc = y[row * ldy + c];
+    float u = 0.f;
+#pragma unroll
+    for (int t = 0; t < STREAMS_MAX; ++t) {
+      if (t < n) {
+        float acc = 0.f;
+#pragma unroll
+        for (int s = 0; s < STREAMS_MAX; ++s)
+          if (s < n) acc = fmaf(sm[s * n + t], old[s], acc);
+        acc = fmaf(wo[t], yc, acc);
+        xs[t * plane + row * width + c] = acc;
+        u = fmaf(wn[t], acc, u);
+      }
+    }
+    ss = fmaf(u, u, ss);
+  }
+  if (!next_in) return;
+  ss = block_sum_256(ss, sh);      // (the barrier inside also orders this workgroup's writes before its reads below)
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(width) + eps);
+  for (int c = threadIdx.x; c < width; c += 256) {
+    float u = 0.f;
+    for (int t = 0; t < n; ++t) u = fmaf(wn[t], xs[t * plane + row * width + c], u);
+    u *= inv;
+    store_as(out, row * ldo + c, out_dt, g ? u * g[c] : u);
   }
 }
 
@@ -629,13 +793,13 @@ int dn_concat_cast(const float* a, long long lda, int wa, const float* b, long l
   return dn_launch_status();
 }
 
-int dn_conv_rows(const float* h, long long ldh, const float* w, const float* hist, const int* row_start, const int* slots, int S, int T,
+int dn_conv_rows(const float* h, long long ldh, const float* w, const float* bias, const float* hist, const int* row_start, const int* slots, int S, int T,
                  int width, int taps, int identity, int silu, void* out, int out_dt, long long ldo, long long hist_stride,
                  hipStream_t stream) {
   if (!float_kind(out_dt)) return DN_ERR_DTYPE;
   if (taps < 1 || S < 1 || ldh < width || ldo < width) return DN_ERR_SHAPE;
   if (T == 0) return 0;
-  hipLaunchKernelGGL(conv_rows_kernel, dim3(T), dim3(256), 0, stream, h, static_cast<size_t>(ldh), w, hist, row_start, slots, S, width,
+  hipLaunchKernelGGL(conv_rows_kernel, dim3(T), dim3(256), 0, stream, h, static_cast<size_t>(ldh), w, bias, hist, row_start, slots, S, width,
                      taps, identity, silu, out, out_dt, static_cast<size_t>(ldo), static_cast<size_t>(hist_stride));
   return dn_launch_status();
 }
@@ -726,21 +890,21 @@ int dn_gated(const void* x, int x_dt, long long ldx, const float* g, long long l
 int dn_state_scan(const float* r, long long ldr, const float* k, long long ldk, const float* v, long long ldv, const float* w,
                   long long ldw, const float* u, const float* beta, long long ldb, const float* w_head, int G, float* state,
                   long long slot_stride, const int* row_start, const int* slots, int S, int T, int H, int dk, int dv, int mode,
-                  int key_from_decay, int beta_logits, float* out, long long ldo, hipStream_t stream) {
+                  int key_from_decay, int beta_logits, int w_rows, float* out, long long ldo, hipStream_t stream) {
   if (dk < 1 || dk > 256 || dv < 1 || H < 1 || G < 1 || H % G != 0) return DN_ERR_SHAPE;
-  if (!key_from_decay && k == nullptr) return DN_ERR_SHAPE;
+  if ((!key_from_decay && k == nullptr) || (w_rows && (w == nullptr || key_from_decay))) return DN_ERR_SHAPE;
   if (mode < SCAN_BEFORE || mode > SCAN_DELTA || (mode == SCAN_DELTA && beta == nullptr) || (w == nullptr) == (w_head == nullptr))
     return DN_ERR_SHAPE;
   if (S == 0) return 0;
   const int read_after = mode;
   ScanArgs a{r, k, v, w, u, beta, w_head, static_cast<size_t>(ldr), static_cast<size_t>(ldk), static_cast<size_t>(ldv),
-             static_cast<size_t>(ldw), static_cast<size_t>(ldb), G, state, static_cast<size_t>(slot_stride), row_start, slots, H, dk, dv, read_after, key_from_decay, beta_logits, out,
+             static_cast<size_t>(ldw), static_cast<size_t>(ldb), G, state, static_cast<size_t>(slot_stride), row_start, slots, H, dk, dv, read_after, key_from_decay, beta_logits, w_rows, out,
              static_cast<size_t>(ldo)};
   // (the parts of a column's sum by the head's size alone, never by the step: a row's bits are the same in every step)
   const dim3 few((dv + 15) / 16, H, S), many((dv + 3) / 4, H, S);
   auto by16 = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-  const bool vec = dk % 4 == 0 && dv % 4 == 0 && ldr % 4 == 0 && ldv % 4 == 0 && (w == nullptr || ldw % 4 == 0) &&
-                   (key_from_decay || ldk % 4 == 0) && by16(r) && by16(v) && by16(w) && (key_from_decay || by16(k));
+  const bool vec = dk % 4 == 0 && dv % 4 == 0 && ldr % 4 == 0 && ldv % 4 == 0 && (w == nullptr || w_rows || ldw % 4 == 0) &&
+                   (key_from_decay || ldk % 4 == 0) && by16(r) && by16(v) && (w_rows || by16(w)) && (key_from_decay || by16(k));
   const bool few_rows = T <= 2 * S;      // (decoded tokens: a row or two a request)
 #define DN_SCAN3(DK, KG, GRID, AFTER, VEC)                                                                    \
   do {                                                                                                        \
@@ -770,16 +934,60 @@ int dn_state_scan(const float* r, long long ldr, const float* k, long long ldk, 
 }
 
 int dn_head_norm(const float* o, long long ld, const float* weight, int w_stride, float eps, const float* gate, long long ldg,
-                 int gate_kind, void* out, int out_dt, long long ldo, int T, int H, int dv, hipStream_t stream) {
+                 int gate_kind, int gate_first, const float* skip, long long lds, const float* skip_scale, int skip_dim, void* out,
+                 int out_dt, long long ldo, int T, int H, int dv, hipStream_t stream) {
   if (!float_kind(out_dt)) return DN_ERR_DTYPE;
   if (gate && (gate_kind < 0 || gate_kind > ACT_TANH)) return DN_ERR_SHAPE;
+  if (skip && (!skip_scale || skip_dim < 1)) return DN_ERR_SHAPE;
   if (T == 0) return 0;
+  HeadNormArgs a{o, static_cast<size_t>(ld), weight, w_stride, eps, gate, static_cast<size_t>(ldg), gate_kind, gate_first, skip,
+                 static_cast<size_t>(lds), skip_scale, skip_dim, out, out_dt, static_cast<size_t>(ldo), dv};
   if (dv > 256)
-    hipLaunchKernelGGL(head_norm_wide_kernel, dim3(T, H), dim3(256), 0, stream, o, static_cast<size_t>(ld), weight, w_stride, eps, gate,
-                       static_cast<size_t>(ldg), gate_kind, out, out_dt, static_cast<size_t>(ldo), dv);
+    hipLaunchKernelGGL(head_norm_wide_kernel, dim3(T, H), dim3(256), 0, stream, a);
   else
-    hipLaunchKernelGGL(head_norm_kernel, dim3(T, H), dim3(64), 0, stream, o, static_cast<size_t>(ld), weight, w_stride, eps, gate,
-                       static_cast<size_t>(ldg), gate_kind, out, out_dt, static_cast<size_t>(ldo), dv);
+    hipLaunchKernelGGL(head_norm_kernel, dim3(T, H), dim3(64), 0, stream, a);
+  return dn_launch_status();
+}
+
+int dn_step_sizes(const float* z, long long ldz, const float* bias, const float* rate, const float* x, long long ldx, int T, int H, int dv,
+                  float* decay, long long ldd, float* v, long long ldv, hipStream_t stream) {
+  if (H < 1 || dv < 1 || !rate) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(step_sizes_kernel, dim3(T), dim3(256), 0, stream, z, static_cast<size_t>(ldz), bias, rate, x, static_cast<size_t>(ldx),
+                     H, dv, decay, static_cast<size_t>(ldd), v, static_cast<size_t>(ldv));
+  return dn_launch_status();
+}
+
+int dn_gate_scan(const float* a, long long lda, const float* b, long long ldb, const float* g, long long ldg, const float* bias_a,
+                 const float* bias_b, float* state, long long slot_stride, const int* row_start, const int* slots, int S, int width,
+                 void* out, int out_dt, long long ldo, hipStream_t stream) {
+  if (!float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (width < 1 || S > 65535) return DN_ERR_SHAPE;
+  if (S == 0) return 0;
+  hipLaunchKernelGGL(gate_scan_kernel, dim3((width + 63) / 64, S), dim3(64), 0, stream, a, static_cast<size_t>(lda), b,
+                     static_cast<size_t>(ldb), g, static_cast<size_t>(ldg), bias_a, bias_b, state, static_cast<size_t>(slot_stride), row_start,
+                     slots, width, out, out_dt, static_cast<size_t>(ldo));
+  return dn_launch_status();
+}
+
+int dn_streams_read(const float* xs, long long plane, int n, const float* w_in, const float* g, float eps, void* out, int out_dt,
+                    long long ldo, const int* rows, int R, int width, hipStream_t stream) {
+  if (!float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (n < 1 || n > STREAMS_MAX || width < 1) return DN_ERR_SHAPE;
+  if (R == 0) return 0;
+  hipLaunchKernelGGL(streams_read_kernel, dim3(R), dim3(256), 0, stream, xs, static_cast<size_t>(plane), n, w_in, g, eps, out, out_dt,
+                     static_cast<size_t>(ldo), rows, width);
+  return dn_launch_status();
+}
+
+int dn_streams_write(float* xs, long long plane, int n, const float* mix, const float* w_out, const float* y, long long ldy,
+                     const float* next_in, const float* g, float eps, void* out, int out_dt, long long ldo, int T, int width,
+                     hipStream_t stream) {
+  if (next_in && !float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (n < 1 || n > STREAMS_MAX || width < 1 || (next_in && !out)) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(streams_write_kernel, dim3(T), dim3(256), 0, stream, xs, static_cast<size_t>(plane), n, mix, w_out, y,
+                     static_cast<size_t>(ldy), next_in, g, eps, out, out_dt, static_cast<size_t>(ldo), width);
   return dn_launch_status();
 }
 

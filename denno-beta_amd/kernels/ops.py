@@ -102,6 +102,7 @@ def _declare(name, lib):
             "dn_layernorm_join": [P, P, I, c_longlong, P, P, P, P, I, I, F, I, I, P],
             "dn_kv_write": [P, I, I, I, P, P, P, I, I, I, I, I, P],
             "dn_cast": [P, P, c_longlong, I, I, P],
+            "dn_pair_rows": [P, P, P, P, I, P, c_longlong, c_longlong, c_longlong, I, I, P, I, P],
         },
         "gemm": {
             "dn_gemm": [P, I, P, P, P, I, P, I, I, I, I, I, I, I, I, P, c_longlong, P],
@@ -119,6 +120,8 @@ def _declare(name, lib):
             "dn_attention": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, I, P],
             "dn_attention_rows": [P, I, P, I, P, P, P, I, P, P, I, P, I, I, I, I, I, F, I, I, P],
             "dn_attention_rows_tile": [I],
+            "dn_attention_extras": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, I, P, I, I, I, P],
+            "dn_attention_rows_extras": [P, I, P, I, P, P, P, I, P, P, I, P, I, I, I, I, I, F, I, I, P, I, I, I, P],
             "dn_attention_flash": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, P],
             "dn_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, I, F, I, P],
         },
@@ -128,7 +131,7 @@ def _declare(name, lib):
             "dn_rmsnorm_add": [P, I, c_longlong, P, P, F, P, c_longlong, I, I, F, P],
             "dn_depth_mix": [P, c_longlong, I, P, P, c_longlong, P],
             "dn_unit_heads": [P, c_longlong, P, c_longlong, I, I, I, F, F, P],
-            "dn_conv_rows": [P, c_longlong, P, P, P, P, I, I, I, I, I, I, P, I, c_longlong, c_longlong, P],
+            "dn_conv_rows": [P, c_longlong, P, P, P, P, P, I, I, I, I, I, I, P, I, c_longlong, c_longlong, P],
             "dn_history_update": [P, I, c_longlong, P, P, P, I, I, I, c_longlong, P],
             "dn_conv_heads": [P, c_longlong, P, P, P, P, I, I, I, I, I, I, F, F, F, I, I, P, c_longlong, c_longlong, P],
             "dn_rotary_runs": [P, I, c_longlong, P, I, P, P, I, P],
@@ -137,8 +140,12 @@ def _declare(name, lib):
             "dn_activate": [P, c_longlong, P, P, I, P, I, c_longlong, I, I, P],
             "dn_gated": [P, I, c_longlong, P, c_longlong, I, P, I, c_longlong, I, I, P],
             "dn_state_scan": [P, c_longlong, P, c_longlong, P, c_longlong, P, c_longlong, P, P, c_longlong, P, I, P, c_longlong, P, P,
-                              I, I, I, I, I, I, I, I, P, c_longlong, P],
-            "dn_head_norm": [P, c_longlong, P, I, F, P, c_longlong, I, P, I, c_longlong, I, I, I, P],
+                              I, I, I, I, I, I, I, I, I, P, c_longlong, P],
+            "dn_head_norm": [P, c_longlong, P, I, F, P, c_longlong, I, I, P, c_longlong, P, I, P, I, c_longlong, I, I, I, P],
+            "dn_step_sizes": [P, c_longlong, P, P, P, c_longlong, I, I, I, P, c_longlong, P, c_longlong, P],
+            "dn_gate_scan": [P, c_longlong, P, c_longlong, P, c_longlong, P, P, P, c_longlong, P, P, I, I, P, I, c_longlong, P],
+            "dn_streams_read": [P, c_longlong, I, P, P, F, P, I, c_longlong, P, I, I, P],
+            "dn_streams_write": [P, c_longlong, I, P, P, P, c_longlong, P, P, F, P, I, c_longlong, I, I, P],
         },
         "grouped": {
             "dn_heads_linear": [P, I, c_longlong, I, I, P, I, P, I, c_longlong, I, I, I, I, I, I, P],
@@ -265,6 +272,21 @@ def embed_sum(parts, out):
         tables[i], indices[i], rows[i], scales[i] = table.data_ptr(), index.data_ptr(), table.shape[0], float(scale)
     _ok(_lib("elementwise").dn_embed_sum(tables, indices, rows, scales, n, out.data_ptr(), T, E, _CODE[dtype], _stream()),
         "embed")
+    return out
+
+
+def pair_rows(tokens, positions, row_start, slots, last, mul_prev, mul_cur, buckets, out, write=True):
+    """out[t] = (token before * mul_prev + tokens[t] * mul_cur) mod buckets, in 64-bit: the row of a table that the pair (token
+    before, token) picks; a request's first token (positions[t] == 0) takes row `buckets`.  The token before a request's
+    first row of this step is last[slot] (int32 [slots, 1]); with `write` the request's last token of this step is left there."""
+    _dev(tokens, "tokens", _I32, 1), _dev(positions, "positions", _I32, 1), _dev(out, "out", _I32, 1), _dev(last, "last", _I32, 2)
+    T = tokens.shape[0]
+    S = _request_tables(row_start, slots, "pair_rows")
+    _need(tokens.is_contiguous() and positions.is_contiguous() and out.is_contiguous() and positions.shape[0] == T and out.shape[0] == T
+          and last.shape[1] == 1 and buckets >= 1 and mul_prev >= 0 and mul_cur >= 0, "pair_rows: shapes")
+    _ok(_lib("elementwise").dn_pair_rows(tokens.data_ptr(), positions.data_ptr(), row_start.data_ptr(), slots.data_ptr(), S,
+                                         last.data_ptr(), last.stride(0), int(mul_prev), int(mul_cur), int(buckets), int(bool(write)),
+                                         out.data_ptr(), T, _stream()), "pair_rows")
     return out
 
 
@@ -589,7 +611,7 @@ def attention_writes_packed(dtype, page_size, head_dim, single_rows, max_context
 
 
 def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, window=0, tiles_wide=None,
-              single_rows=False, max_context=0, decode_waves=None):
+              single_rows=False, max_context=0, decode_waves=None, chunk=0, bias=None, sink=False):
     """Causal attention of the batch's rows over the paged cache.
 
     q: [T, >= H*dh] rows contiguous, head h at columns h*dh..; out: [T, H*dh];
@@ -599,6 +621,10 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
     tiles_wide: the same rows cut into tiles of up to 128 rows;
     single_rows: a pure decode step: request s brings row s and is tile s, (s or -1, s, 1, position);
     max_context: the longest context then.
+
+    chunk > 0: the row at position p reads only the keys from p // chunk * chunk on (runs of `chunk` positions counted from
+    the request's first); bias: 32-bit [H, span], bias[h, p - key] is added to the scaled score (distances from span on
+    take the last entry); sink: one more summand exp(0) under the softmax (a key with score 0 and no value).
 
     Three kernels: 32-bit takes the plain one; bfloat16 takes the MFMA kernel over tiles_wide, or,
     for a pure decode step, the split kernel (with both, out may be packed rows); a head size that
@@ -622,9 +648,16 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
     _need(1 <= dh <= 256, lambda: f"attention: head size {dh} must be at most 256")
     _need(n_heads % Hkv == 0, lambda: f"attention: {n_heads} heads over {Hkv} key heads")
     ldq, ldo = _rows(q, "q"), (0 if out_packed else _rows(out, "out"))
+    extras = chunk > 0 or bias is not None or bool(sink)
+    span = 0
+    if bias is not None:
+        _dev(bias, "bias", (torch.float32,), 2)
+        _need(bias.is_contiguous() and bias.shape[0] == n_heads and bias.shape[1] >= 1, "attention: bias is [heads, span]")
+        span = bias.shape[1]
+    _need(chunk >= 0, "attention: chunk")
     lib = _lib("attention")
     # (the kernel for portions takes the largest score for the largest product: a scale that is not positive goes the plain way)
-    fast = q.dtype == torch.bfloat16 and ps % 16 == 0 and ldq % 8 == 0 and q.data_ptr() % 16 == 0 and scale > 0
+    fast = q.dtype == torch.bfloat16 and ps % 16 == 0 and ldq % 8 == 0 and q.data_ptr() % 16 == 0 and scale > 0 and not extras
     decode = fast and decode_attention_applies(q.dtype, ps, dh, single_rows, max_context)
     _need(not out_packed or (fast and attention_writes_packed(q.dtype, ps, dh, single_rows, max_context, tiles_wide)),
           "attention: packed rows as out are written by the bfloat16 kernels only")
@@ -681,15 +714,17 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
         _need(n_tiles == T, "attention: a step of single rows has a tile for every row")
         key_tiles = -(-max_context // lib.dn_attention_rows_tile(dh))
         part = torch.empty(n_tiles * n_heads * key_tiles * (dh + 2), dtype=torch.float32, device=q.device)
-        _ok(lib.dn_attention_rows(
+        _ok(lib.dn_attention_rows_extras(
             q.data_ptr(), ldq, out.data_ptr(), ldo, k_pool.data_ptr(), v_pool.data_ptr(), block_tables.data_ptr(),
             block_tables.shape[1], base, base + 12 * n_tiles, n_tiles, part.data_ptr(), int(max_context), n_heads, Hkv,
-            dh, ps, float(scale), int(window), _CODE[q.dtype], _stream()), "attention (single rows)")
+            dh, ps, float(scale), int(window), int(chunk), _ptr(bias), span, int(bool(sink)), _CODE[q.dtype], _stream()),
+            "attention (single rows)")
         return out
-    _ok(lib.dn_attention(
+    _ok(lib.dn_attention_extras(
         q.data_ptr(), ldq, out.data_ptr(), ldo, k_pool.data_ptr(), v_pool.data_ptr(), block_tables.data_ptr(),
         block_tables.shape[1], base, base + 4 * n_tiles, base + 8 * n_tiles, base + 12 * n_tiles, n_tiles,
-        n_heads, Hkv, dh, ps, float(scale), int(window), _CODE[q.dtype], _stream()), "attention")
+        n_heads, Hkv, dh, ps, float(scale), int(window), int(chunk), _ptr(bias), span, int(bool(sink)), _CODE[q.dtype],
+        _stream()), "attention")
     return out
 
 
@@ -1005,8 +1040,8 @@ def concat_cast(a, b, out):
     return out
 
 
-def conv_rows(h, w, hist, row_start, slots, out, identity=True, act=None):
-    """out[t, c] = act((h[t, c] if identity else 0) + sum_j w[c, j] h[t - taps + 1 + j, c]) inside each request; the rows
+def conv_rows(h, w, hist, row_start, slots, out, identity=True, act=None, bias=None):
+    """out[t, c] = act((h[t, c] if identity else 0) + bias[c] + sum_j w[c, j] h[t - taps + 1 + j, c]) inside each request; the rows
     before a request's first row of this step come from hist [slots, (taps - 1) * width] (oldest first).  h: 32-bit rows whose
     first `width` columns are the channels (width = w.shape[0]); act: None or "silu"."""
     _dev(h, "h", (torch.float32,), 2), _dev(w, "w", (torch.float32,), 2), _dev(out, "out", _FLOATS, 2)
@@ -1015,7 +1050,8 @@ def conv_rows(h, w, hist, row_start, slots, out, identity=True, act=None):
     S = _request_tables(row_start, slots, "conv_rows")
     _need(h.shape[1] >= width and w.is_contiguous() and tuple(out.shape) == (T, width) and act in (None, "silu"), "conv_rows: shapes")
     stride = _history(hist, (taps - 1) * width, "conv_rows") if taps > 1 else 0
-    _ok(_lib("sequence").dn_conv_rows(h.data_ptr(), _rows(h, "h"), w.data_ptr(), _ptr(hist) if taps > 1 else 0, row_start.data_ptr(),
+    _f32vec(bias, "bias", width)
+    _ok(_lib("sequence").dn_conv_rows(h.data_ptr(), _rows(h, "h"), w.data_ptr(), _ptr(bias), _ptr(hist) if taps > 1 else 0, row_start.data_ptr(),
                                       slots.data_ptr(), S, T, width, taps, int(bool(identity)), int(act == "silu"), out.data_ptr(),
                                       _CODE[out.dtype], _rows(out, "out"), stride, _stream()),
         "conv_rows")
@@ -1137,22 +1173,24 @@ def gated(x, g, kind, out):
 
 
 def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, read_after=False, key_from_decay=False, beta=None,
-               w_head=None, qk_heads=None, beta_logits=False):
+               w_head=None, qk_heads=None, beta_logits=False, w_rows=False):
     """The recurrence of a matrix state per head, S [dk, dv], over each request's rows of this step in order:
       a = 1 - w if key_from_decay else k
       read_after:  S <- diag(w) S + a v^T ;  o = S^T r
       beta given:  S <- diag(w) S ;  e = beta (v - S^T a) ;  S <- S + a e^T ;  o = S^T r        (the delta rule)
       else:        o = (S + diag(u) a v^T)^T r ;  S <- diag(w) S + a v^T        (u None: no bonus)
     r, k: 32-bit [T, qk_heads * dk] (qk_heads None: n_heads; fewer: head h reads head h // (n_heads // qk_heads));
-    w: 32-bit [T, heads * dk], or None with w_head: 32-bit [heads], one decay per head for every row and channel;
+    w: 32-bit [T, heads * dk], or (w_rows) [T, heads], one decay per row and head for all the head's channels, or None with
+    w_head: 32-bit [heads], one decay per head for every row and channel;
     v, out: 32-bit [T, heads * dv]; beta: 32-bit [T, heads] (beta_logits: it holds z, and beta is 1 / (1 + e^-z)); state: 32-bit [slots, heads * dv * dk] (a head's state
     held [value column][key channel]), read and written at the requests' slots."""
     G = n_heads if qk_heads is None else qk_heads
     _need(G >= 1 and n_heads % G == 0, lambda: f"state_scan: {n_heads} heads over {G} heads of queries and keys")
     _need((w is None) != (w_head is None), "state_scan: a decay per row and channel (w) or one per head (w_head)")
-    _need(not (key_from_decay and w is None), "state_scan: keys from the decay need w")
+    _need(not (key_from_decay and (w is None or w_rows)), "state_scan: keys from the decay need w per channel")
+    _need(not w_rows or w is not None, "state_scan: w_rows needs w")
     given = ((r, "r", G * dk), (v, "v", n_heads * dv), (out, "out", n_heads * dv)) + (() if key_from_decay else ((k, "k", G * dk),)) \
-        + (() if w is None else ((w, "w", n_heads * dk),)) + (() if beta is None else ((beta, "beta", n_heads),))
+        + (() if w is None else ((w, "w", n_heads if w_rows else n_heads * dk),)) + (() if beta is None else ((beta, "beta", n_heads),))
     for t, name, n in given:
         _dev(t, name, (torch.float32,), 2)
         _need(t.shape[1] == n, lambda: f"state_scan: {name} {tuple(t.shape)}")
@@ -1169,14 +1207,15 @@ def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, rea
                                        _rows(w, "w") if w is not None else 0, _ptr(u), _ptr(beta),
                                        _rows(beta, "beta") if beta is not None else 0, _ptr(w_head), G, state.data_ptr(), stride,
                                        row_start.data_ptr(), slots.data_ptr(), S, T, n_heads, dk, dv, mode, int(key_from_decay),
-                                       int(bool(beta_logits)), out.data_ptr(), _rows(out, "out"), _stream()),
+                                       int(bool(beta_logits)), int(bool(w_rows)), out.data_ptr(), _rows(out, "out"), _stream()),
         "state_scan" if beta is None else "state_scan (delta rule)")
     return out
 
 
-def head_norm(o, weight, eps, out, n_heads, gate=None, gate_kind="silu"):
-    """out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight * act(gate[t, h, :]).  weight: None, one per
-    column of o, or one per column of a head (shared by the heads); o and gate 32-bit."""
+def head_norm(o, weight, eps, out, n_heads, gate=None, gate_kind="silu", gate_first=False, skip=None, skip_scale=None):
+    """y = o (+ skip * skip_scale, a second summand [T, n] with a number per run of n / len(skip_scale) columns); gate_first: y
+    times act(gate) before the norm, else behind it; out[t, h, :] = y[t, h, :] / sqrt(mean(y[t, h, :]^2) + eps) * weight.
+    weight: None, one per column of o, or one per column of a head (shared by the heads); o, gate and skip 32-bit."""
     _dev(o, "o", (torch.float32,), 2), _dev(out, "out", _FLOATS, 2)
     T, n = o.shape
     _need(n % n_heads == 0 and tuple(out.shape) == (T, n), "head_norm: shapes")
@@ -1189,9 +1228,94 @@ def head_norm(o, weight, eps, out, n_heads, gate=None, gate_kind="silu"):
     if gate is not None:
         _dev(gate, "gate", (torch.float32,), 2)
         _need(tuple(gate.shape) == (T, n) and gate_kind in ("silu", "sigmoid", "tanh"), "head_norm: gate")
+    skip_dim = 0
+    if skip is not None:
+        _dev(skip, "skip", (torch.float32,), 2), _f32vec(skip_scale, "skip_scale")
+        _need(tuple(skip.shape) == (T, n) and skip_scale is not None and skip_scale.numel() >= 1 and n % skip_scale.numel() == 0,
+              "head_norm: skip")
+        skip_dim = n // skip_scale.numel()
     _ok(_lib("sequence").dn_head_norm(o.data_ptr(), _rows(o, "o"), _ptr(weight), w_stride, float(eps), _ptr(gate),
-                                      _rows(gate, "gate") if gate is not None else 0, ACTIVATIONS[gate_kind], out.data_ptr(),
-                                      _CODE[out.dtype], _rows(out, "out"), T, n_heads, dv, _stream()), "head_norm")
+                                      _rows(gate, "gate") if gate is not None else 0, ACTIVATIONS[gate_kind], int(bool(gate_first)),
+                                      _ptr(skip), _rows(skip, "skip") if skip is not None else 0, _ptr(skip_scale), skip_dim,
+                                      out.data_ptr(), _CODE[out.dtype], _rows(out, "out"), T, n_heads, dv, _stream()), "head_norm")
+    return out
+
+
+def step_sizes(z, bias, rate, x, n_heads, decay, v):
+    """dt = log(1 + e^(z[t, h] + bias[h])); decay[t, h] = exp(-rate[h] * dt); v[t, h, :] = dt * x[t, h, :]: what a recurrence with
+    one decay per head and token reads.  z [T, heads], x and v [T, heads * dv], decay [T, heads]; all 32-bit."""
+    for t, name in ((z, "z"), (x, "x"), (decay, "decay"), (v, "v")):
+        _dev(t, name, (torch.float32,), 2)
+    T, n = x.shape
+    _need(n % n_heads == 0 and z.shape == (T, n_heads) and decay.shape == (T, n_heads) and v.shape == (T, n), "step_sizes: shapes")
+    _f32vec(bias, "bias", n_heads), _f32vec(rate, "rate", n_heads)
+    _ok(_lib("sequence").dn_step_sizes(z.data_ptr(), _rows(z, "z"), _ptr(bias), rate.data_ptr(), x.data_ptr(), _rows(x, "x"), T, n_heads,
+                                       n // n_heads, decay.data_ptr(), _rows(decay, "decay"), v.data_ptr(), _rows(v, "v"), _stream()),
+        "step_sizes")
+    return decay, v
+
+
+def gate_scan(a, b, g, bias_a, bias_b, state, row_start, slots, out):
+    """A recurrence of single numbers over each request's rows in order: z = sigmoid(a + bias_a); u = b + bias_b;
+    c = u + 1/2 where u >= 0, sigmoid(u) below; S <- (1 - z) S + z c; out = S * silu(g).  a, b, g: 32-bit [T, width] (columns of
+    wider rows); state: 32-bit [slots, width]; out [T, width]."""
+    for t, name in ((a, "a"), (b, "b"), (g, "g")):
+        _dev(t, name, (torch.float32,), 2)
+    _dev(out, "out", _FLOATS, 2)
+    T, width = a.shape
+    S = _request_tables(row_start, slots, "gate_scan")
+    _need(b.shape == (T, width) and g.shape == (T, width) and out.shape == (T, width), "gate_scan: shapes")
+    _f32vec(bias_a, "bias_a", width), _f32vec(bias_b, "bias_b", width)
+    stride = _history(state, width, "gate_scan")
+    _ok(_lib("sequence").dn_gate_scan(a.data_ptr(), _rows(a, "a"), b.data_ptr(), _rows(b, "b"), g.data_ptr(), _rows(g, "g"), _ptr(bias_a),
+                                      _ptr(bias_b), state.data_ptr(), stride, row_start.data_ptr(), slots.data_ptr(), S, width,
+                                      out.data_ptr(), _CODE[out.dtype], _rows(out, "out"), _stream()), "gate_scan")
+    return out
+
+
+STREAMS_MAX = 8
+
+
+def _streams(xs, what):
+    _dev(xs, "xs", (torch.float32,), 3)
+    n, T, width = xs.shape
+    _need(xs.is_contiguous() and 1 <= n <= STREAMS_MAX, lambda: f"{what}: 1 to {STREAMS_MAX} copies of the stream, contiguous")
+    return n, T, width
+
+
+def streams_read(xs, w_in, weight, eps, out, rows=None):
+    """xs: the stream as n copies, 32-bit [n, T, width].  u = sum_s w_in[s] xs[s] (w_in None: the plain sum); out[r] =
+    u[rows[r]] / sqrt(mean(u^2) + eps) * weight (weight: a number per column or None; eps None: no norm, u itself)."""
+    n, T, width = _streams(xs, "streams_read")
+    _dev(out, "out", _FLOATS, 2)
+    _f32vec(w_in, "w_in", n), _f32vec(weight, "weight", width)
+    R = out.shape[0]
+    if rows is not None:
+        _dev(rows, "rows", _I32, 1)
+        _need(rows.is_contiguous() and rows.shape[0] == R, "streams_read: rows")
+    else:
+        _need(R == T, "streams_read: out rows")
+    _need(out.shape[1] == width, "streams_read: out")
+    _ok(_lib("sequence").dn_streams_read(xs.data_ptr(), T * width, n, _ptr(w_in), _ptr(weight), -1.0 if eps is None else float(eps),
+                                         out.data_ptr(), _CODE[out.dtype], _rows(out, "out"), _ptr(rows), R, width, _stream()),
+        "streams_read")
+    return out
+
+
+def streams_write(xs, y, mix, w_out, next_in=None, weight=None, eps=0.0, out=None):
+    """Every copy anew from the old ones and a sublayer's result: xs[t] <- sum_s mix[s, t] xs[s] + w_out[t] * y, in place.
+    next_in given: the same kernel then reads the new copies as streams_read(xs, next_in, weight, eps, out) does."""
+    n, T, width = _streams(xs, "streams_write")
+    _dev(y, "y", (torch.float32,), 2)
+    _need(tuple(y.shape) == (T, width), "streams_write: y")
+    _f32vec(mix, "mix", n * n), _f32vec(w_out, "w_out", n), _f32vec(next_in, "next_in", n), _f32vec(weight, "weight", width)
+    if next_in is not None:
+        _dev(out, "out", _FLOATS, 2)
+        _need(tuple(out.shape) == (T, width), "streams_write: out")
+    _ok(_lib("sequence").dn_streams_write(xs.data_ptr(), T * width, n, mix.data_ptr(), w_out.data_ptr(), y.data_ptr(), _rows(y, "y"),
+                                          _ptr(next_in), _ptr(weight), float(eps), _ptr(out) if next_in is not None else 0,
+                                          _CODE[out.dtype] if next_in is not None else 0,
+                                          _rows(out, "out") if next_in is not None else 0, T, width, _stream()), "streams_write")
     return out
 
 

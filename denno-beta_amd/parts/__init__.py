@@ -1,7 +1,7 @@
-from .base import (ARRANGEMENTS, FEED_FORWARDS, FILTERS, MIXERS, NORMS, POSITIONS, DeferredSum, FixedState, PagedKV, Part, Runtime)
-from . import blocks, feedforward, filters, mixers, norms, positions, recurrent   # noqa: F401  (registers the parts)
+from .base import (ARRANGEMENTS, CONNECTORS, FEED_FORWARDS, FILTERS, MIXERS, NORMS, POSITIONS, DeferredSum, FixedState, PagedKV, Part, Runtime)
+from . import blocks, connectors, feedforward, filters, mixers, norms, positions, recurrent   # noqa: F401  (registers the parts)
 from .linear import Linear
 from .model import CacheView, DecoderModel, DecoderSpec, EmbeddingTable, LayerCall, LayerSpec
 
-__all__ = ["ARRANGEMENTS", "FEED_FORWARDS", "FILTERS", "MIXERS", "NORMS", "POSITIONS", "DeferredSum", "FixedState", "PagedKV", "Part",
+__all__ = ["ARRANGEMENTS", "CONNECTORS", "FEED_FORWARDS", "FILTERS", "MIXERS", "NORMS", "POSITIONS", "DeferredSum", "FixedState", "PagedKV", "Part",
            "Runtime", "Linear", "CacheView", "DecoderModel", "DecoderSpec", "EmbeddingTable", "LayerCall", "LayerSpec"]

@@ -11,6 +11,8 @@ Kinds of part and their registries:
   feed-forward     FEED_FORWARDS   forward(h, ctx, accumulate_into)
   norm             NORMS           forward(x, out_dtype, rows=None) -> tensor
   input filter     FILTERS         forward(h, ctx, cache) -> what the mixer reads ; cache_spec()
+  connector        CONNECTORS      read(xs, norm, out_dtype) -> what a sublayer reads of several copies of the stream;
+                                   write(xs, y): the copies anew from a sublayer's result
   position code    POSITIONS       table() for the embedding stage, rotate(q, k, ctx) for mixers
   arrangement      ARRANGEMENTS    SLOTS names its parts and their kinds; forward(x, ctx, caches, runtime): how
                                    norms, mixers and feed-forwards stand in a block
@@ -75,6 +77,10 @@ class Runtime:
     deferred_sums: bool = True             # EngineOptions.deferred_sums
     # a product's sum that is not in the stream yet (DeferredSum): the next norm's kernel adds it, or the model does
     stream_deferred: Optional["DeferredSum"] = None
+    # a stream kept as several copies (the "multi_stream" arrangement): the (connector, norm) with which the block that runs
+    # next reads it first (set by the model), and the rows that the block before has read for this one in its last write's kernel
+    next_read: Optional[tuple] = None
+    stream_rows: Optional[torch.Tensor] = None
 
 
 class Part:
@@ -91,6 +97,12 @@ class Part:
 
     def bind(self, tensors: Dict[str, torch.Tensor], runtime: Runtime) -> None:
         self.runtime = runtime
+
+    def cache_parts(self):
+        """The parts that keep a cache or a state each, in the order in which a LayerCall lists their caches: the part
+        itself, or, for a mixer made of several (parts.mixers.ParallelMixers), those; such a mixer's forward then
+        takes a list of CacheViews."""
+        return [self]
 
     def packed_input(self, n_rows: int) -> bool:
         """A mixer or feed-forward whose first product takes packed rows (kernels.ops.PackedMatrix)
@@ -197,5 +209,6 @@ NORMS = Registry("norm")
 POSITIONS = Registry("position encoding")
 ARRANGEMENTS = Registry("block arrangement")
 FILTERS = Registry("input filter")
+CONNECTORS = Registry("connector")
 # the kinds that an arrangement's SLOTS may name
-KINDS = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "filter": FILTERS}
+KINDS = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "filter": FILTERS, "connector": CONNECTORS}

@@ -119,6 +119,31 @@ class FilteredPreNormBlock:
             self.ffn.forward(self.norm2.forward(x, runtime.act_dtype), ctx, accumulate_into=x)
 
 
+@ARRANGEMENTS.register("pre_norm_plain")
+class PlainPreNormBlock:
+    """x += mixer(norm1(x)); x += ffn(norm2(x)), every norm a kernel of its own.  The mixer may be several side by side
+    (its `cache_parts`: a call of this block then names a cache for each).  A block whose feed-forward is "none" ends after
+    the mixer."""
+
+    SLOTS = {"norm1": "norm", "mixer": "mixer", "norm2": "norm", "ffn": "feed_forward"}
+
+    def __init__(self, norm1, mixer, norm2, ffn):
+        self.norm1, self.mixer, self.norm2, self.ffn = norm1, mixer, norm2, ffn
+        self.has_ffn = not getattr(ffn, "absent", False)
+
+    def parts(self):
+        return [self.norm1, self.mixer] + ([self.norm2, self.ffn] if self.has_ffn else [])
+
+    def mixers(self):
+        return self.mixer.cache_parts()
+
+    def forward(self, x, ctx, caches, runtime):
+        runtime.stream_stats = None
+        self.mixer.forward(self.norm1.forward(x, runtime.act_dtype), ctx, caches if len(caches) != 1 else caches[0], accumulate_into=x)
+        if self.has_ffn:
+            self.ffn.forward(self.norm2.forward(x, runtime.act_dtype), ctx, accumulate_into=x)
+
+
 @ARRANGEMENTS.register("sandwich")
 class SandwichBlock:
     """A norm before and a norm behind each sublayer: x += post1(mixer(norm1(x))); x += post2(ffn(norm2(x))).  The norms
@@ -157,3 +182,49 @@ class SandwichBlock:
         if self.has_ffn:
             h = self.norm2.forward(x, runtime.act_dtype)
             self.post2.add_into(self._result(self.ffn, x, h, ctx), x)
+
+
+@ARRANGEMENTS.register("multi_stream")
+class MultiStreamBlock:
+    """The stream is several copies (DecoderSpec.streams).  For each sublayer f (the mixer, then the feed-forward) with its
+    connector c and norm: y = f(norm(c.read(copies))); c.write(copies, y) makes every copy anew.  A block whose
+    feed-forward is "none" ends after the mixer.  A sublayer's result comes as 32-bit rows of its own (`returns_rows`, or
+    added into rows of zeros).  The read of the sublayer that follows, in this block or the next, runs in the kernel of
+    the write before it: the rows travel in `runtime.stream_rows`."""
+
+    SLOTS = {"norm1": "norm", "hc1": "connector", "mixer": "mixer", "norm2": "norm", "hc2": "connector", "ffn": "feed_forward"}
+    multi_stream = True
+
+    def __init__(self, norm1, hc1, mixer, norm2, hc2, ffn):
+        self.norm1, self.hc1, self.mixer, self.norm2, self.hc2, self.ffn = norm1, hc1, mixer, norm2, hc2, ffn
+        self.has_ffn = not getattr(ffn, "absent", False)
+
+    def parts(self):
+        return [self.norm1, self.hc1, self.mixer] + ([self.norm2, self.hc2, self.ffn] if self.has_ffn else [])
+
+    def mixers(self):
+        return self.mixer.cache_parts()
+
+    def first_read(self):
+        """(connector, norm) of the sublayer that reads the stream first."""
+        return self.hc1, self.norm1
+
+    def forward(self, xs, ctx, caches, runtime):
+        act = runtime.act_dtype
+        runtime.stream_stats = None
+        came = getattr(runtime, "stream_rows", None)      # (the block before read for this one as it wrote)
+        runtime.stream_rows = None
+        h = came if came is not None else self.hc1.read(xs, self.norm1, act)
+        cache = caches if len(caches) != 1 else caches[0]
+        y = SandwichBlock._result(self.mixer, xs[0], h, ctx, cache)
+        nxt = getattr(runtime, "next_read", None)
+        if self.has_ffn:
+            h = self.hc1.write(xs, y, self.hc2, self.norm2, act)
+            y = SandwichBlock._result(self.ffn, xs[0], h, ctx)
+            last = self.hc2
+        else:
+            last = self.hc1
+        if nxt is not None:
+            runtime.stream_rows = last.write(xs, y, nxt[0], nxt[1], act)
+        else:
+            last.write(xs, y)

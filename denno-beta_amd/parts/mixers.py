@@ -1,6 +1,8 @@
 """Mixers: the parts that let a token see other tokens."""
 from __future__ import annotations
 
+import math
+
 import torch
 
 from ..kernels import ops
@@ -268,3 +270,137 @@ class LatentAttention(Part):
         og = torch.empty((T, self.o_width), dtype=act, device=dev)
         ops.gated(o, z[:, gate:], "sigmoid", og)
         self.out(og, residual=accumulate_into)
+
+
+def distance_buckets(n_distances: int, n_buckets: int, far: float):
+    """The bucket of every distance 0 .. n_distances - 1: a bucket each below half the buckets; from there on the buckets are
+    spaced evenly in the logarithm of the distance up to `far`; the last bucket takes everything beyond."""
+    half = n_buckets // 2
+    out = []
+    for n in range(n_distances):
+        if n < half or half == 0:
+            out.append(min(n, n_buckets - 1))
+        else:
+            out.append(min(n_buckets - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (n_buckets - half)))))
+    return out
+
+
+@MIXERS.register("chunk_attention")
+class ChunkAttention(Part):
+    """Causal softmax attention inside chunks, without a rotation, whose values are the keys' projection.
+
+    q = W_q h and k = W_k h are each normed as one vector over all heads (x / sqrt(mean(x^2) + eps) times a weight per
+    entry); the values are k as projected, before that norm.  score(i, j) = q_i . k_j * scale * temp[head] + rel[bucket(i - j),
+    head], with `distance_buckets` over the table's rows; position i reads j <= i of its own run of `chunk` positions
+    (runs counted from the sequence's position 0); a sink (score 0, no value) stands under the softmax if `sink`.
+    Query head a reads key head a // (n_heads // n_kv_heads).  Then the output projection.
+
+    The temperature rides on the queries' norm weight; the bias is a table by distance, made once (a row sees distances
+    below `chunk` only), that the attention kernels add to the scaled score."""
+    graph_safe = True
+    returns_rows = True
+    libraries = ("sequence",)
+
+    def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float, chunk: int, n_buckets: int,
+                 bias_far: float, eps: float, names: dict, sink: bool = True):
+        """names: q, k, o (matrices); q_norm, k_norm (vectors over all heads); rel [n_buckets, heads]; temp [heads]."""
+        if n_heads % n_kv_heads != 0:
+            raise ValueError(f"chunk_attention: {n_heads} heads cannot share {n_kv_heads} key heads")
+        if not 1 <= head_dim <= 256:
+            raise ValueError(f"chunk_attention: head size {head_dim}: the attention kernels take head sizes up to 256")
+        if chunk < 1 or n_buckets < 1 or not bias_far > max(1, n_buckets // 2):
+            raise ValueError(f"chunk_attention: chunk {chunk}, {n_buckets} buckets up to a distance of {bias_far}")
+        self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim
+        self.scale, self.chunk, self.n_buckets, self.bias_far, self.eps = float(scale), int(chunk), int(n_buckets), float(bias_far), eps
+        self.sink, self.names = bool(sink), dict(names)
+        self.q_width, self.kv_width = n_heads * head_dim, n_kv_heads * head_dim
+        self.proj = Linear(width, self.q_width + self.kv_width, names["q"] + "+k", None, init_std=width ** -0.5,
+                           weight_sources=((names["q"], self.q_width), (names["k"], self.kv_width)))
+        self.out = Linear(self.q_width, width, names["o"], None, init_std=self.q_width ** -0.5)
+
+    def param_specs(self):
+        n = self.names
+        return self.proj.param_specs() + self.out.param_specs() + [
+            ParamSpec(n["q_norm"], (self.q_width,), "vector", ("normal", 1.0, 0.1)),
+            ParamSpec(n["k_norm"], (self.kv_width,), "vector", ("normal", 1.0, 0.1)),
+            ParamSpec(n["rel"], (self.n_buckets, self.n_heads), "vector", ("normal", 0.0, 0.5)),
+            ParamSpec(n["temp"], (self.n_heads,), "vector", ("normal", 1.0, 0.2))]
+
+    def cache_spec(self):
+        return PagedKV(self.n_kv_heads, self.head_dim)
+
+    def bind(self, tensors, runtime):
+        super().bind(tensors, runtime)
+        self.proj.bind(tensors), self.out.bind(tensors)
+        n = self.names
+        temp = tensors[n["temp"]].to(torch.float32)
+        self.q_norm = (tensors[n["q_norm"]].to(torch.float32) * temp.repeat_interleave(self.head_dim)).contiguous()
+        self.k_norm = tensors[n["k_norm"]].contiguous()
+        rows = torch.tensor(distance_buckets(self.chunk, self.n_buckets, self.bias_far), dtype=torch.long, device=temp.device)
+        self.bias = tensors[n["rel"]].to(torch.float32)[rows].t().contiguous()      # [heads, chunk]
+        self.no_freq = torch.empty(0, dtype=torch.float32, device=runtime.device)
+
+    def forward(self, h, ctx, cache, accumulate_into):
+        act, T, dev = self.runtime.act_dtype, h.shape[0], h.device
+        H, G, d, qw, kw = self.n_heads, self.n_kv_heads, self.head_dim, self.q_width, self.kv_width
+        g = ctx.groups[cache.group]
+        z = self.proj(h, out_dtype=torch.float32)
+        q = torch.empty((T, qw), dtype=act, device=dev)
+        kv = torch.empty((T, 2 * kw), dtype=act, device=dev)      # normed keys at column 0, the projection as values at kw
+        ops.rmsnorm(z[:, :qw], self.q_norm, self.eps, q)
+        ops.rmsnorm(z[:, qw:], self.k_norm, self.eps, kv[:, :kw])
+        ops.rotary(z, kv, ctx.positions, self.no_freq, G, 0, d, src_off=qw, dst_off=kw)      # (moved, not turned)
+        if cache.writes:
+            ops.kv_write(kv, 0, kw, g.slot_map, cache.k, cache.v)
+        o = torch.empty((T, qw), dtype=act, device=dev)
+        ops.attention(q, o, cache.k, cache.v, g.block_tables, g.tiles, H, self.scale, 0, tiles_wide=g.tiles_wide,
+                      single_rows=g.single_rows, max_context=g.max_context, chunk=self.chunk, bias=self.bias, sink=self.sink)
+        if accumulate_into is None:
+            return self.out(o, out_dtype=torch.float32)
+        self.out(o, residual=accumulate_into)
+
+
+@MIXERS.register("parallel_mixers")
+class ParallelMixers(Part):
+    """Several mixers side by side that read the same rows; each result is normed over the width (without a mean, with a
+    weight per column of its own) and the result is their mean.  branches: [(kind name, arguments)] of mixers that can
+    return their result as rows (`returns_rows`); every branch keeps a cache or state of its own, so a LayerCall of a
+    layer with this mixer lists one cache per branch."""
+    returns_rows = True
+
+    def __init__(self, width: int, eps: float, branches, norm_names):
+        if len(branches) < 1 or len(branches) != len(norm_names):
+            raise ValueError("parallel_mixers: a norm weight's name for every branch")
+        self.width, self.eps, self.norm_names = width, eps, list(norm_names)
+        self.branches = [MIXERS.make(tuple(b)) for b in branches]
+        for b in self.branches:
+            if not getattr(b, "returns_rows", False):
+                raise TypeError(f"parallel_mixers: {type(b).__name__} cannot return its result as rows")
+        self.graph_safe = all(getattr(b, "graph_safe", False) for b in self.branches)
+        self.libraries = tuple(sorted({"sequence"} | {lib for b in self.branches for lib in getattr(b, "libraries", ())}))
+
+    def cache_parts(self):
+        return list(self.branches)
+
+    def param_specs(self):
+        specs = [ParamSpec(n, (self.width,), "vector", ("normal", 1.0, 0.1)) for n in self.norm_names]
+        for b in self.branches:
+            specs += b.param_specs()
+        return specs
+
+    def bind(self, tensors, runtime):
+        super().bind(tensors, runtime)
+        for b in self.branches:
+            b.bind(tensors, runtime)
+        self.norms = [tensors[n] for n in self.norm_names]
+
+    def forward(self, h, ctx, caches, accumulate_into):
+        if not isinstance(caches, (list, tuple)):
+            caches = [caches]
+        y = accumulate_into
+        if y is None:
+            y = torch.zeros((h.shape[0], self.width), dtype=torch.float32, device=h.device)
+        share = 1.0 / len(self.branches)
+        for b, w, cache in zip(self.branches, self.norms, caches):
+            ops.rmsnorm_add(b.forward(h, ctx, cache, accumulate_into=None), w, None, share, self.eps, y)
+        return y if accumulate_into is None else None

@@ -48,11 +48,14 @@ class LayerCall:
 @dataclass
 class EmbeddingTable:
     """A further table [rows, width] whose rows are added to the token and position rows in the embedding kernel.
-    index: which per-row integers of the step pick its rows: "tokens" or "positions" (fields of StepContext)."""
+    index: which per-row integers of the step pick its rows: "tokens" or "positions" (fields of StepContext), or "pairs":
+    row (token before * pair[0] + token * pair[1]) mod pair[2], and row pair[2], the table's last, for a request's first
+    token; the token before a step's first is then a state of the request (one int32), kept like a mixer's."""
     name: str                     # checkpoint name
     rows: int
     index: str = "tokens"
     scale: float = 1.0
+    pair: Optional[Tuple[int, int, int]] = None     # index "pairs": (multiplier of the token before, of the token, buckets)
 
 
 @dataclass
@@ -72,6 +75,9 @@ class DecoderSpec:
     embedding_scale: float = 1.0          # the token table's rows times this, before the position table's
     extra_embeddings: List[EmbeddingTable] = field(default_factory=list)   # added behind them, in this order
     embedding_norm: Optional[PartSpec] = None   # a norm of the embedded rows, before the first layer
+    # > 0: the stream is kept as this many copies, all equal to the embedding stage's output at the start and added up
+    # behind the last layer; every layer is then of an arrangement that works on copies ("multi_stream")
+    streams: int = 0
     # name -> checkpoint name of a matrix [width, 2 width]: where a LayerCall names it, the stream becomes
     # W [x ; x0], x the stream as it stands and x0 the embedding stage's output (a loop's way back in)
     injections: Dict[str, str] = field(default_factory=dict)
@@ -104,8 +110,11 @@ class DecoderModel:
         self.embedding = TokenEmbedding(spec.vocab, spec.width, spec.token_table)
         self.position = POSITIONS.make(spec.position)
         for t in spec.extra_embeddings:
-            if t.index not in ("tokens", "positions"):
-                raise ValueError(f"embedding table {t.name!r}: rows are picked by 'tokens' or 'positions', not {t.index!r}")
+            if t.index not in ("tokens", "positions", "pairs"):
+                raise ValueError(f"embedding table {t.name!r}: rows are picked by 'tokens', 'positions' or 'pairs', not {t.index!r}")
+            if t.index == "pairs" and (t.pair is None or len(t.pair) != 3 or t.pair[2] < 1 or t.pair[2] + 1 != t.rows
+                                       or min(t.pair[:2]) < 0):
+                raise ValueError(f"embedding table {t.name!r}: pairs need (multiplier, multiplier, buckets) with buckets + 1 = rows")
         if len(spec.extra_embeddings) > ops.EMBED_TABLES_MAX - 2:
             raise ValueError(f"{len(spec.extra_embeddings)} further embedding tables; the kernel adds up {ops.EMBED_TABLES_MAX} in all")
         self.extra_tables = {}
@@ -124,6 +133,18 @@ class DecoderModel:
         # the head: a matrix of its own, or the token table, transposed
         self.head = Linear(spec.width, spec.vocab, spec.head_weight or spec.token_table, spec.head_bias)
         self._check_run_order()
+        # the states of the embedding stage (the token before, for tables picked by pairs) are caches behind the layers'
+        self.pair_caches = {}
+        for t in spec.extra_embeddings:
+            if t.index == "pairs":
+                self.pair_caches[t.name] = self.n_caches
+                self.cache_specs.append(FixedState((1,), "int32"))
+                self.n_caches += 1
+        many = [bool(getattr(b, "multi_stream", False)) for b in self.blocks]
+        if spec.streams < 0 or (spec.streams > 0) != all(many) or (spec.streams == 0 and any(many)):
+            raise ValueError("DecoderSpec.streams > 0 goes with layers of a multi-stream arrangement, all of them, and only with those")
+        if spec.streams > 0 and (spec.injections or spec.embedding_norm is not None or any(c.average or c.inject for c in spec.run_order)):
+            raise ValueError("a stream kept as several copies has no injections, averages over depth or embedding norm")
         self.runtime = None
         self.graph_safe = all(getattr(p, "graph_safe", False) for p in self.all_parts())
 
@@ -234,7 +255,11 @@ class DecoderModel:
         rt = self.runtime
         order = self.spec.run_order
         kept = None
-        if self.averages:
+        xs = None
+        if self.spec.streams:
+            xs = torch.empty((self.spec.streams, ctx.T, self.spec.width), dtype=torch.float32, device=rt.device)
+            x = xs[0]
+        elif self.averages:
             # every call's result is kept, plane j + 1 for call j behind the embedding stage's in plane 0; a call works in
             # its own plane, which holds what went on from the call before
             kept = torch.empty((len(order) + 2, ctx.T, self.spec.width), dtype=torch.float32, device=rt.device)
@@ -248,7 +273,14 @@ class DecoderModel:
             parts = [(self.embedding.weight, ctx.tokens, self.spec.embedding_scale)]
             if self.position.table() is not None:
                 parts.append((self.position.table(), ctx.positions, 1.0))
-            parts += [(self.extra_tables[t.name], getattr(ctx, t.index), t.scale) for t in self.spec.extra_embeddings]
+            for t in self.spec.extra_embeddings:
+                if t.index == "pairs":
+                    picked = ops.pair_rows(ctx.tokens, ctx.positions, ctx.row_start, ctx.state_slots,
+                                           cache.view(self.pair_caches[t.name], True).state, t.pair[0], t.pair[1], t.pair[2],
+                                           torch.empty_like(ctx.tokens))
+                else:
+                    picked = getattr(ctx, t.index)
+                parts.append((self.extra_tables[t.name], picked, t.scale))
             ops.embed_sum(parts, x)
         rt.stream_stats = rt.stream_deferred = None      # nobody has left anything for a norm of these rows yet
         if self.embedding_norm is not None:
@@ -258,7 +290,15 @@ class DecoderModel:
             if x.data_ptr() != kept[0].data_ptr():
                 kept[0].copy_(x)
             x = ops.depth_mix(kept, 1, self._one, kept[1])
+        if xs is not None:
+            xs[1:].copy_(x)      # (every copy starts as the embedding stage's output)
+            rt.stream_rows = None
         for i, call in enumerate(order):
+            if xs is not None:
+                nxt = self.blocks[order[i + 1].layer] if i + 1 < len(order) else None
+                rt.next_read = nxt.first_read() if nxt is not None else None
+                self.blocks[call.layer].forward(xs, ctx, [cache.view(c, call.writes_cache) for c in call.caches()], rt)
+                continue
             if call.inject is not None:
                 if rt.stream_deferred is not None:
                     rt.stream_deferred.flush(x)
@@ -287,7 +327,17 @@ class DecoderModel:
         rt.next_takes_deferred = False
         if ctx.R == 0:
             return torch.empty((0, self.spec.vocab), dtype=torch.float32, device=rt.device)
-        h = self.final_norm.forward(x, rt.act_dtype, rows=ctx.logit_rows, packed=self.head.packed_input(ctx.R))
+        if xs is not None:
+            # the copies are added up; a norm without a mean runs in the same kernel, on the wanted rows alone
+            fn = self.final_norm
+            if getattr(fn, "kind_name", None) == "rmsnorm":
+                h = ops.streams_read(xs, None, fn.weight, fn.eps, torch.empty((ctx.R, self.spec.width), dtype=rt.act_dtype, device=rt.device),
+                                     rows=ctx.logit_rows)
+            else:
+                x = ops.streams_read(xs, None, None, None, torch.empty((ctx.T, self.spec.width), dtype=torch.float32, device=rt.device))
+                h = fn.forward(x, rt.act_dtype, rows=ctx.logit_rows, packed=self.head.packed_input(ctx.R))
+        else:
+            h = self.final_norm.forward(x, rt.act_dtype, rows=ctx.logit_rows, packed=self.head.packed_input(ctx.R))
         logits = self.head(h, out_dtype=torch.float32)
         if self.spec.logit_scale != 1.0 or self.spec.logit_softcap > 0:
             ops.logits_post(logits, self.spec.logit_scale, self.spec.logit_softcap)

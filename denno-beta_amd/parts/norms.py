@@ -52,19 +52,22 @@ class LayerNorm(Part):
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Part):
-    """x / sqrt(mean(x^2) + eps) * weight, eps inside the root, statistics in 32-bit."""
+    """x / sqrt(mean(x^2) + eps) * weight, eps inside the root, statistics in 32-bit.  one_weight: the checkpoint holds a
+    single number (a tensor without dimensions) that multiplies every column."""
     graph_safe = True
     libraries = ("sequence",)
 
-    def __init__(self, width: int, eps: float, weight_name: str):
-        self.width, self.eps, self.weight_name = width, eps, weight_name
+    def __init__(self, width: int, eps: float, weight_name: str, one_weight: bool = False):
+        self.width, self.eps, self.weight_name, self.one_weight = width, eps, weight_name, bool(one_weight)
 
     def param_specs(self):
-        return [ParamSpec(self.weight_name, (self.width,), "vector", ("normal", 1.0, 0.1))]
+        return [ParamSpec(self.weight_name, () if self.one_weight else (self.width,), "vector", ("normal", 1.0, 0.1))]
 
     def bind(self, tensors, runtime):
         super().bind(tensors, runtime)
         self.weight = tensors[self.weight_name]
+        if self.one_weight:      # (the kernels take a number per column)
+            self.weight = self.weight.reshape(1).expand(self.width).contiguous()
 
     def forward(self, x, out_dtype, rows=None, packed=False):
         # (packed rows are not written here: the consumer's Linear takes a tensor as well)

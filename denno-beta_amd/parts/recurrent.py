@@ -261,3 +261,120 @@ class ChannelDelta(Part):
         if accumulate_into is None:
             return self.out(y, out_dtype=F32)
         self.out(y, residual=accumulate_into)
+
+
+@MIXERS.register("min_gru")
+class MinGRU(Part):
+    """A recurrence of single numbers whose gates read the token alone: z = sigmoid(W_z h + b_z); u = W_x h + b_x; the
+    candidate is u + 1/2 where u >= 0 and sigmoid(u) below; S_t = (1 - z) S_(t-1) + z * candidate; the result is
+    W_o (S_t * silu(W_g h)).  State: S, `inner` numbers in 32-bit."""
+    graph_safe = True
+    returns_rows = True
+    libraries = ("sequence",)
+
+    def __init__(self, width: int, inner: int, names: dict):
+        """names: z, x, g, o (matrices); z_bias, x_bias (vectors)."""
+        self.width, self.inner, self.names = width, inner, dict(names)
+        n = names
+        # one product for everything that reads h; its 32-bit result feeds the recurrence (the biases are added there)
+        self.proj = Linear(width, 3 * inner, n["z"] + "+x+g", None, init_std=width ** -0.5,
+                           weight_sources=((n["z"], inner), (n["x"], inner), (n["g"], inner)))
+        self.out = Linear(inner, width, n["o"], None, init_std=inner ** -0.5)
+
+    def param_specs(self):
+        return self.proj.param_specs() + self.out.param_specs() + [
+            ParamSpec(self.names["z_bias"], (self.inner,), "vector", ("normal", 0.0, 1.0)),
+            ParamSpec(self.names["x_bias"], (self.inner,), "vector", ("normal", 0.0, 0.5))]
+
+    def cache_spec(self):
+        return FixedState((self.inner,))
+
+    def bind(self, tensors, runtime):
+        super().bind(tensors, runtime)
+        self.proj.bind(tensors), self.out.bind(tensors)
+        self.z_bias, self.x_bias = tensors[self.names["z_bias"]], tensors[self.names["x_bias"]]
+
+    def forward(self, h, ctx, cache, accumulate_into):
+        n = self.inner
+        z = self.proj(h, out_dtype=F32)
+        y = torch.empty((h.shape[0], n), dtype=self.runtime.act_dtype, device=h.device)
+        ops.gate_scan(z[:, :n], z[:, n:2 * n], z[:, 2 * n:], self.z_bias, self.x_bias, cache.state, ctx.row_start, ctx.state_slots, y)
+        if accumulate_into is None:
+            return self.out(y, out_dtype=F32)
+        self.out(y, residual=accumulate_into)
+
+
+@MIXERS.register("mamba2")
+class Mamba2(Part):
+    """A state-space mixer with one decay per head and token.  W_in h is laid out [z: inner | x: inner | B: groups * N |
+    C: groups * N | dt: heads], inner = heads * value_dim.  x, B and C pass a short causal convolution per channel (with a
+    bias) and silu; dt = log(1 + e^(dt + dt_bias)).  Per head (head a reads B and C of group a // (heads // groups)):
+    S <- exp(-e^(A_log) dt) S + dt B x^T (S is N x value_dim), y = S^T C + D x.  y times silu(z) is normed without a mean in
+    `norm_groups` equal parts, times a weight per column; then the output projection.  State: S in 32-bit and the
+    convolution's last taps - 1 inputs."""
+    graph_safe = True
+    returns_rows = True
+    libraries = ("sequence",)
+
+    def __init__(self, width: int, n_heads: int, value_dim: int, state_dim: int, n_groups: int, taps: int, norm_groups: int,
+                 eps: float, names: dict):
+        """names: in, o (matrices); conv [channels, taps], conv_bias, dt_bias, A_log, D, norm."""
+        if n_heads % n_groups != 0:
+            raise ValueError(f"mamba2: {n_heads} heads cannot share {n_groups} groups of B and C")
+        inner = n_heads * value_dim
+        if norm_groups < 1 or inner % norm_groups != 0:
+            raise ValueError(f"mamba2: {inner} columns cannot be normed in {norm_groups} equal parts")
+        if taps < 1:
+            raise ValueError(f"mamba2: {taps} taps")
+        self.width, self.n_heads, self.value_dim, self.state_dim, self.n_groups = width, n_heads, value_dim, state_dim, n_groups
+        self.taps, self.norm_groups, self.eps, self.names = taps, norm_groups, eps, dict(names)
+        self.inner, self.bc = inner, n_groups * state_dim
+        self.channels = inner + 2 * self.bc
+        self.proj = Linear(width, 2 * inner + 2 * self.bc + n_heads, names["in"], None, init_std=width ** -0.5)
+        self.out = Linear(inner, width, names["o"], None, init_std=inner ** -0.5)
+
+    def param_specs(self):
+        n = self.names
+        return self.proj.param_specs() + self.out.param_specs() + [
+            ParamSpec(n["conv"], (self.channels, self.taps), "vector", ("normal", 0.0, 0.4)),
+            ParamSpec(n["conv_bias"], (self.channels,), "vector", ("normal", 0.0, 0.1)),
+            ParamSpec(n["dt_bias"], (self.n_heads,), "vector", ("normal", -1.0, 1.0)),
+            ParamSpec(n["A_log"], (self.n_heads,), "vector", ("uniform", -2.0, 0.5)),
+            ParamSpec(n["D"], (self.n_heads,), "vector", ("normal", 1.0, 0.3)),
+            ParamSpec(n["norm"], (self.inner,), "vector", ("normal", 1.0, 0.1))]
+
+    def cache_spec(self):
+        return FixedState((self.inner * self.state_dim + (self.taps - 1) * self.channels,))
+
+    def bind(self, tensors, runtime):
+        super().bind(tensors, runtime)
+        self.proj.bind(tensors), self.out.bind(tensors)
+        n = self.names
+        self.conv, self.conv_bias = tensors[n["conv"]].contiguous(), tensors[n["conv_bias"]]
+        self.dt_bias, self.skip, self.norm = tensors[n["dt_bias"]], tensors[n["D"]], tensors[n["norm"]]
+        self.rate = torch.exp(tensors[n["A_log"]].to(F32)).contiguous()
+
+    def forward(self, h, ctx, cache, accumulate_into):
+        act, T, dev = self.runtime.act_dtype, h.shape[0], h.device
+        H, inner, bc, C = self.n_heads, self.inner, self.bc, self.channels
+        n_state = inner * self.state_dim
+        state, past = cache.state[:, :n_state], cache.state[:, n_state:]
+        proj = self.proj(h, out_dtype=F32)
+        gate, raw, dt = proj[:, :inner], proj[:, inner:inner + C], proj[:, inner + C:]
+        xbc = torch.empty((T, C), dtype=F32, device=dev)
+        ops.conv_rows(raw, self.conv, past, ctx.row_start, ctx.state_slots, xbc, identity=False, act="silu", bias=self.conv_bias)
+        if self.taps > 1 and cache.writes:
+            ops.history_update(raw, past, ctx.row_start, ctx.state_slots)
+        x, B, Cm = xbc[:, :inner], xbc[:, inner:inner + bc], xbc[:, inner + bc:]
+        decay = torch.empty((T, H), dtype=F32, device=dev)
+        v = torch.empty((T, inner), dtype=F32, device=dev)
+        ops.step_sizes(dt, self.dt_bias, self.rate, x, H, decay, v)
+        o = torch.empty((T, inner), dtype=F32, device=dev)
+        ops.state_scan(Cm, B, v, decay, None, state, ctx.row_start, ctx.state_slots, H, self.state_dim, self.value_dim, o,
+                       read_after=True, qk_heads=self.n_groups, w_rows=True)
+        y = torch.empty((T, inner), dtype=act, device=dev)
+        ops.head_norm(o, self.norm, self.eps, y, self.norm_groups, gate=gate, gate_kind="silu", gate_first=True, skip=x,
+                      skip_scale=self.skip)
+        if accumulate_into is None:
+            return self.out(y, out_dtype=F32)
+        self.out(y, residual=accumulate_into)

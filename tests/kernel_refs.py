@@ -129,7 +129,7 @@ def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None, n
 
 
 def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, window=0, tiles_wide=None,
-              single_rows=False, max_context=0, decode_waves=None):
+              single_rows=False, max_context=0, decode_waves=None, chunk=0, bias=None, sink=False):
     n_pages, hkv, ps, dh = k_pool.shape
     group = n_heads // hkv
     tl = tiles.cpu().tolist()
@@ -141,6 +141,8 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
         for i in range(nrows):
             pos = pos0 + i
             lo = max(0, pos - window + 1) if window > 0 else 0
+            if chunk > 0:
+                lo = max(lo, pos // chunk * chunk)
             keys = torch.arange(lo, pos + 1)
             pages = bt[seq][keys // ps].long()
             offs = keys % ps
@@ -149,7 +151,13 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
                 k = kf[pages, h // group, offs, :]                  # [n, dh]
                 v = vf[pages, h // group, :, offs]
                 qv = q[row0 + i, h * dh:(h + 1) * dh].float()
-                p = torch.softmax((k @ qv) * scale, dim=0)
+                sc = (k @ qv) * scale
+                if bias is not None:
+                    sc = sc + bias[h][torch.clamp(pos - keys, max=bias.shape[1] - 1)]
+                if sink:      # (a key with score 0 and no value)
+                    p = torch.softmax(torch.cat([sc, sc.new_zeros(1)]), dim=0)[:-1]
+                else:
+                    p = torch.softmax(sc, dim=0)
                 out[row0 + i, h * dh:(h + 1) * dh] = (p @ v).to(out.dtype)
     return out
 
@@ -289,7 +297,7 @@ def _requests(row_start, slots):
     return [(sl[s], rs[s], rs[s + 1]) for s in range(len(sl)) if sl[s] >= 0]
 
 
-def conv_rows(h, w, hist, row_start, slots, out, identity=True, act=None):
+def conv_rows(h, w, hist, row_start, slots, out, identity=True, act=None, bias=None):
     width, taps = w.shape
     h = h[:, :width]
     res = torch.zeros((h.shape[0], width), dtype=torch.float32)
@@ -297,6 +305,8 @@ def conv_rows(h, w, hist, row_start, slots, out, identity=True, act=None):
         rows = h[a:b] if taps == 1 else torch.cat([hist[slot].view(taps - 1, width), h[a:b]], dim=0)
         for t in range(b - a):
             acc = h[a + t].clone() if identity else torch.zeros(width)
+            if bias is not None:
+                acc = acc + bias
             for j in range(taps):
                 acc += w[:, j] * rows[t + j]
             res[a + t] = acc
@@ -366,7 +376,7 @@ def gated(x, g, kind, out):
 
 
 def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, read_after=False, key_from_decay=False, beta=None,
-               w_head=None, qk_heads=None, beta_logits=False):
+               w_head=None, qk_heads=None, beta_logits=False, w_rows=False):
     H = n_heads
     if beta is not None and beta_logits:
         beta = torch.sigmoid(beta)
@@ -376,7 +386,7 @@ def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, rea
         S = state[slot].view(H, dv, dk).transpose(1, 2).clone()      # (held [head][value column][key channel])
         for t in range(a, b):
             rt, vt = spread(r[t]), v[t].view(H, dv)
-            wt = w[t].view(H, dk) if w is not None else w_head.view(H, 1).expand(H, dk)
+            wt = (w[t].view(H, 1).expand(H, dk) if w_rows else w[t].view(H, dk)) if w is not None else w_head.view(H, 1).expand(H, dk)
             at = (1.0 - wt) if key_from_decay else spread(k[t])
             kv = at[:, :, None] * vt[:, None, :]
             if beta is not None:
@@ -395,17 +405,82 @@ def state_scan(r, k, v, w, u, state, row_start, slots, n_heads, dk, dv, out, rea
     return out
 
 
-def head_norm(o, weight, eps, out, n_heads, gate=None, gate_kind="silu"):
+def head_norm(o, weight, eps, out, n_heads, gate=None, gate_kind="silu", gate_first=False, skip=None, skip_scale=None):
     T, n = o.shape
     dv = n // n_heads
-    y = o.view(T, n_heads, dv)
+    y = o
+    if skip is not None:
+        y = y + skip * skip_scale.repeat_interleave(n // skip_scale.numel())
+    if gate is not None and gate_first:
+        y = y * _act(gate_kind, gate)
+    y = y.reshape(T, n_heads, dv)
     y = y / torch.sqrt((y * y).mean(dim=-1, keepdim=True) + eps)
     if weight is not None:
         y = y * (weight.view(n_heads, dv) if weight.numel() == n else weight)
     y = y.reshape(T, n)
-    if gate is not None:
+    if gate is not None and not gate_first:
         y = y * _act(gate_kind, gate)
     out.copy_(y)
+    return out
+
+
+def step_sizes(z, bias, rate, x, n_heads, decay, v):
+    T, n = x.shape
+    dt = torch.nn.functional.softplus(z.double() + (bias.double() if bias is not None else 0.0))
+    decay.copy_(torch.exp(-rate.double() * dt))
+    v.copy_((dt[:, :, None] * x.double().view(T, n_heads, n // n_heads)).reshape(T, n))
+    return decay, v
+
+
+def gate_scan(a, b, g, bias_a, bias_b, state, row_start, slots, out):
+    z = torch.sigmoid(a.double() + (bias_a.double() if bias_a is not None else 0.0))
+    u = b.double() + (bias_b.double() if bias_b is not None else 0.0)
+    cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    gate = _act("silu", g.double())
+    for slot, lo, hi in _requests(row_start, slots):
+        S = state[slot].double().clone()
+        for t in range(lo, hi):
+            S = (1 - z[t]) * S + z[t] * cand[t]
+            out[t] = (S * gate[t]).to(out.dtype)
+        state[slot] = S.to(state.dtype)
+    return out
+
+
+def streams_read(xs, w_in, weight, eps, out, rows=None):
+    n = xs.shape[0]
+    u = sum((w_in[s].double() if w_in is not None else 1.0) * xs[s].double() for s in range(n))
+    if rows is not None:
+        u = u[rows.long()]
+    if eps is not None:
+        u = u / torch.sqrt((u * u).mean(dim=-1, keepdim=True) + eps)
+    if weight is not None:
+        u = u * weight.double()
+    out.copy_(u)
+    return out
+
+
+def streams_write(xs, y, mix, w_out, next_in=None, weight=None, eps=0.0, out=None):
+    n = xs.shape[0]
+    old = xs.double().clone()
+    m = mix.double().view(n, n)
+    for t in range(n):
+        xs[t] = (sum(m[s, t] * old[s] for s in range(n)) + w_out[t].double() * y.double()).to(xs.dtype)
+    if next_in is not None:
+        streams_read(xs, next_in, weight, eps, out)
+    return out
+
+
+def pair_rows(tokens, positions, row_start, slots, last, mul_prev, mul_cur, buckets, out, write=True):
+    tok = tokens.tolist()
+    out.fill_(buckets)
+    for slot, lo, hi in _requests(row_start, slots):
+        for t in range(lo, hi):
+            if int(positions[t]) == 0:
+                continue
+            prev = tok[t - 1] if t > lo else int(last[slot, 0])
+            out[t] = (prev * mul_prev + tok[t] * mul_cur) % buckets
+        if write:
+            last[slot, 0] = tok[hi - 1]
     return out
 
 
