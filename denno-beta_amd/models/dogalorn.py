@@ -77,11 +77,10 @@ def _check_layer(i, layer, layers):
         read_int(mlp, "ff", minimum=1)
     src = read_int(layer, "weights_of", default=None, minimum=0)
     if src is not None:
-        if src >= len(layers) or not isinstance(layers[src], dict) or layers[src].get("weights_of") is not None or src == i:
-            raise ConfigError(f"{where}.weights_of = {src}: it names a layer with tensors of its own")
-        other = {k: v for k, v in layers[src].items() if k != "weights_of"}
-        if other != {k: v for k, v in layer.items() if k != "weights_of"}:
-            raise ConfigError(f"{where}: a layer that runs with layer {src}'s tensors has that layer's sizes")
+        if src >= len(layers) or src == i or not isinstance(layers[src], dict) or layers[src].get("weights_of") is not None:
+            raise ConfigError(f"{where}.weights_of = {src}: it must name another layer, one with tensors of its own")
+        if layers[src].get("type") != kind or (layers[src].get("mlp") is None) != (mlp is None):
+            raise ConfigError(f"{where}: a layer that runs with layer {src}'s tensors is of that layer's type, with or without a feed-forward as it")
 
 
 @dataclass(frozen=True)

@@ -132,4 +132,4 @@ def write_safetensors(path: str, layout: Iterable[Tuple[str, torch.dtype, Tuple[
                 raise SafetensorsError(f"'{name}': produced {t.dtype}{list(t.shape)}, "
                                        f"layout says {dtype}{list(shape)}")
             t = t.contiguous().cpu()
-            f.write(t.view(torch.uint8).numpy().tobytes() if t.numel() else b"")
+            f.write(t.reshape(-1).view(torch.uint8).numpy().tobytes() if t.numel() else b"")

@@ -1059,3 +1059,41 @@ def test_few_rows_product_with_an_inner_size_below_64(M, K):
         want = res + exact
         o.linear(a, wp, bias, residual=res)
         assert torch.allclose(res, want, **TOL[torch.bfloat16]), (M, N, K)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,Hkv,dh,ps,chunk,span", [(4, 2, 16, 16, 24, 24), (8, 8, 96, 16, 200, 200), (3, 1, 24, 8, 13, 13), (2, 2, 64, 16, 1, 1),
+                                                    (2, 1, 128, 32, 64, 64), (5, 5, 80, 16, 300, 300), (2, 2, 64, 16, 0, 50),
+                                                    (4, 4, 64, 16, 128, 128), (2, 2, 256, 16, 100, 100)])
+def test_attention_in_chunks_with_a_bias_by_distance_and_a_sink(dtype, H, Hkv, dh, ps, chunk, span):
+    """Every kernel that `attention` may take (portions in tiles of 16 and of 128 rows, single rows) with chunks, a bias by
+    distance and a sink, each alone and all together: a decoded token deep in a context, a whole prompt, a portion that
+    starts inside a chunk, a first token."""
+    seq_lens, new_rows = [300, 70, 133, 1, 430], [1, 70, 21, 1, 300]
+    q, k, v, bt, tiles, T = paged_case(seq_lens, new_rows, H, Hkv, dh, ps, dtype, seed=H + dh + chunk)
+    scale = 1 / math.sqrt(dh)
+    bias = torch.randn(H, span, generator=torch.Generator().manual_seed(chunk)).to(DEV)
+    qs = q[:, :H * dh]
+    for kw in (dict(chunk=chunk), dict(bias=bias), dict(sink=True), dict(chunk=chunk, bias=bias, sink=True)):
+        if kw.get("chunk") == 0 and len(kw) == 1:
+            continue
+        want = R.attention(qs, torch.zeros(T, H * dh, device=DEV), k, v, bt, tiles, H, scale, 0, **kw)
+        out = torch.zeros(T, H * dh, dtype=dtype, device=DEV)
+        ops().attention(qs, out, k, v, bt, tiles, H, scale, 0, **kw)
+        assert torch.allclose(out.float(), want, **TOL[dtype]), ("tiles of 16", kw.keys())
+        out = torch.zeros(T, H * dh, dtype=dtype, device=DEV)
+        ops().attention(qs, out, k, v, bt, tiles, H, scale, 0, tiles_wide=paged_case.wide, **kw)
+        assert torch.allclose(out.float(), want, **TOL[dtype]), ("tiles of 128", kw.keys())
+    # a step of single rows: contexts on both sides of a chunk's edge, of a page's and of a split's
+    seq_lens = [1, chunk or 17, (chunk or 17) + 1, 256, 257, 700, 1024, 2 * (chunk or 17)]
+    q, k, v, bt, tiles, T = paged_case(seq_lens, [1] * len(seq_lens), H, Hkv, dh, ps, dtype, seed=dh + span)
+    qs = q[:, :H * dh]
+    kw = dict(chunk=chunk, bias=bias, sink=True)
+    want = R.attention(qs, torch.zeros(T, H * dh, device=DEV), k, v, bt, tiles, H, scale, 0, **kw)
+    out = torch.zeros(T, H * dh, dtype=dtype, device=DEV)
+    ops().attention(qs, out, k, v, bt, tiles, H, scale, 0, tiles_wide=paged_case.wide, single_rows=True, max_context=1024, **kw)
+    assert torch.allclose(out.float(), want, **TOL[dtype])
+    if dtype == torch.float32 and dh % 16 == 0:      # the kernels for single rows and for portions: the same bits
+        rows = torch.zeros(T, H * dh, dtype=dtype, device=DEV)
+        ops().attention(qs, rows, k, v, bt, tiles, H, scale, 0, **kw)
+        assert torch.equal(rows, out)

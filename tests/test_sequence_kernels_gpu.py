@@ -406,3 +406,104 @@ def test_a_row_does_not_depend_on_its_neighbours():
     many = ops.heads_linear(a, w, torch.zeros(50, H * N, device=DEV))
     one = ops.heads_linear(a[17:18].contiguous(), w, torch.zeros(1, H * N, device=DEV))
     assert torch.equal(many[17:18], one)
+
+
+# ---- a convolution's bias, a decay per row and head, a gate before the norm, a recurrence of single numbers, a stream in copies ----
+@pytest.mark.parametrize("taps", [1, 3, 4])
+def test_conv_with_a_bias(taps):
+    width = 29
+    row_start, slots, T = tables([2, 9, 1, 4], [1, 3, -1, 0])
+    h = torch.randn(T, width + 6, device=DEV)
+    w = torch.randn(width, taps, device=DEV)
+    b = torch.randn(width, device=DEV)
+    hist = torch.randn(4, max(taps - 1, 1) * width, device=DEV)
+    both("conv_rows", lambda: (h, w, hist, row_start, slots, torch.zeros(T, width, device=DEV), False, "silu", b), [5])
+
+
+@pytest.mark.parametrize("dk,dv,heads,groups", [(16, 8, 4, 2), (48, 48, 6, 1), (24, 12, 3, 3), (128, 64, 2, 1), (6, 10, 2, 1)])
+@pytest.mark.parametrize("lengths", [[1, 1, 1], [5, 40, 1, 17]])
+def test_state_scan_with_a_decay_per_row_and_head(dk, dv, heads, groups, lengths):
+    row_start, slots, T = tables(lengths, list(range(len(lengths)))[::-1])
+    g = torch.Generator(device=DEV).manual_seed(dk * 7 + dv)
+    rnd = lambda *s: torch.randn(*s, device=DEV, generator=g)      # noqa: E731
+    r, k, v = rnd(T, groups * dk), rnd(T, groups * dk), rnd(T, heads * dv)
+    w = torch.sigmoid(rnd(T, heads) + 2.0)
+    state0 = rnd(len(lengths), heads * dk * dv) * 0.3
+
+    def make():
+        return (r, k, v, w, None, state0.clone(), row_start, slots, heads, dk, dv, torch.zeros(T, heads * dv, device=DEV), True, False, None,
+                None, groups, False, True)
+    both("state_scan", make, [5, 11])
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("heads,dv", [(2, 24), (1, 300), (4, 16)])
+def test_head_norm_with_the_gate_first_and_a_second_summand(dtype, heads, dv):
+    T, n = 9, heads * dv
+    o, gate, skip = torch.randn(T, n, device=DEV), torch.randn(T, n, device=DEV), torch.randn(T, n, device=DEV)
+    w = torch.randn(n, device=DEV)
+    for parts in (1, 2, n // 4):
+        scale = torch.randn(parts, device=DEV)
+        both("head_norm", lambda: (o, w, 1e-5, torch.empty(T, n, dtype=dtype, device=DEV), heads, gate, "silu", True, skip, scale), [3], dtype)
+    both("head_norm", lambda: (o, w, 1e-5, torch.empty(T, n, dtype=dtype, device=DEV), heads, gate, "sigmoid", False, skip, scale), [3], dtype)
+    both("head_norm", lambda: (o, None, 1e-5, torch.empty(T, n, dtype=dtype, device=DEV), heads, gate, "silu", True), [3], dtype)
+
+
+def test_step_sizes():
+    T, H, dv = 11, 3, 10
+    z = torch.randn(T, H + 4, device=DEV) * 4
+    x = torch.randn(T, H * dv + 2, device=DEV)
+    bias, rate = torch.randn(H, device=DEV), torch.rand(H, device=DEV) * 3
+    both("step_sizes", lambda: (z[:, 2:2 + H], bias, rate, x[:, :H * dv], H, torch.empty(T, H, device=DEV), torch.empty(T, H * dv, device=DEV)),
+         [5, 6])
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("lengths", [[1, 1, 1, 1], [3, 70, 1, 9, 8]])
+@pytest.mark.parametrize("width", [5, 64, 200])
+def test_gate_scan(dtype, lengths, width):
+    row_start, slots, T = tables(lengths, [3, 0, -1, 2, 1][:len(lengths)])
+    z = torch.randn(T, 3 * width + 1, device=DEV) * 2
+    ba, bb = torch.randn(width, device=DEV), torch.randn(width, device=DEV)
+    state0 = torch.randn(4, width, device=DEV)
+
+    def make():
+        return (z[:, :width], z[:, width:2 * width], z[:, 2 * width:3 * width], ba, bb, state0.clone(), row_start, slots,
+                torch.zeros(T, width, dtype=dtype, device=DEV))
+    both("gate_scan", make, [5, 8], dtype)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("n,width", [(1, 40), (3, 256), (4, 77), (8, 1030)])
+def test_a_stream_in_copies_read_and_written(dtype, n, width):
+    T = 7
+    xs = torch.randn(n, T, width, device=DEV)
+    w_in, w_out, mix = torch.randn(n, device=DEV), torch.randn(n, device=DEV), torch.randn(n, n, device=DEV)
+    g = torch.randn(width, device=DEV)
+    y = torch.randn(T, width, device=DEV)
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    both("streams_read", lambda: (xs, w_in, g, 1e-5, torch.empty(T, width, dtype=dtype, device=DEV)), [4], dtype)
+    both("streams_read", lambda: (xs, None, g, 1e-5, torch.empty(3, width, dtype=dtype, device=DEV), rows), [4], dtype)
+    both("streams_read", lambda: (xs, None, None, None, torch.empty(T, width, device=DEV)), [4])
+    both("streams_write", lambda: (xs.clone(), y, mix, w_out), [0])
+    both("streams_write", lambda: (xs.clone(), y, mix, w_out, w_in, g, 1e-6, torch.empty(T, width, dtype=dtype, device=DEV)), [0, 7], dtype)
+    # the write that also reads gives what the two kernels give one after the other, bit for bit
+    a, b = xs.clone(), xs.clone()
+    one = ops.streams_write(a, y, mix, w_out, w_in, g, 1e-6, torch.empty(T, width, dtype=dtype, device=DEV))
+    ops.streams_write(b, y, mix, w_out)
+    two = ops.streams_read(b, w_in, g, 1e-6, torch.empty(T, width, dtype=dtype, device=DEV))
+    assert torch.equal(a, b) and torch.equal(one, two)
+
+
+def test_rows_picked_by_pairs_of_tokens():
+    row_start, slots, T = tables([1, 6, 2, 3], [2, 0, -1, 1])
+    tokens = torch.randint(0, 50000, (T,), dtype=torch.int32, device=DEV)
+    positions = torch.tensor([0, 0, 1, 2, 3, 4, 5, 0, 0, 7, 8, 9], dtype=torch.int32, device=DEV)
+    last0 = torch.randint(0, 50000, (3, 1), dtype=torch.int32, device=DEV)
+    for write in (True, False):
+        last_d, last_h = last0.clone(), last0.cpu().clone()
+        got = ops.pair_rows(tokens, positions, row_start, slots, last_d, 1000003, 999983, 30011, torch.empty(T, dtype=torch.int32, device=DEV), write)
+        want = ref.pair_rows(tokens.cpu(), positions.cpu(), row_start.cpu(), slots.cpu(), last_h, 1000003, 999983, 30011,
+                             torch.empty(T, dtype=torch.int32), write)
+        assert torch.equal(got.cpu()[:7], want[:7]) and torch.equal(got.cpu()[9:], want[9:]) and torch.equal(last_d.cpu(), last_h)
+        assert got.cpu()[7:9].tolist() == [30011, 30011]      # (padding at position 0: the table's last row, no state touched)
