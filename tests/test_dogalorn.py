@@ -130,12 +130,12 @@ BOUND = {"float32": 2e-5, "bfloat16": 0.06}
 BF16_OVER, BF16_WORST = 0.02, 0.15
 
 
-def assert_rows(got, want, dtype, what, bound=None):
+def assert_rows(got, want, dtype, what, bound=None, worst=BF16_WORST):
     e = row_errors(got, want)
     b = bound or BOUND[dtype]
     if dtype == "bfloat16" and bound is None:
         over = int((e > b).sum())
-        assert over <= max(1, BF16_OVER * len(e)) and e.max() <= BF16_WORST, (
+        assert over <= max(1, BF16_OVER * len(e)) and e.max() <= worst, (
             f"{what}: {over} of {len(e)} positions are off by more than {b} of their row's spread, the worst (position "
             f"{int(e.argmax())}) by {e.max().item():.3g}")
         return
@@ -389,7 +389,7 @@ def imprint(tensors):
     u, m, g = _directions(tensors, 2)
     n = tensors["l0.mix.right.z"].shape[0]
     tensors["l0.mix.right.z"] = torch.outer(torch.ones(n), 6.0 * m)
-    tensors["l0.mix.right.z.b"] = torch.full((n,), -5.0)
+    tensors["l0.mix.right.z.b"] = torch.full((n,), -7.0)
     tensors["l0.mix.right.x"] = tensors["l0.mix.right.x"] + torch.outer(torch.rand(n, generator=g) + 0.5, 3.0 * m)
     tensors["l0.mix.right.out"] = tensors["l0.mix.right.out"] * 3.0
     tensors["l0.mix.left.out"] = tensors["l0.mix.left.out"] * 0.2
@@ -411,7 +411,7 @@ FAR = {"attention": (config([with_mlp(parallel(2, 1, 16, 64, 8, far=100, buckets
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_far_tokens_count(backend, folders, what, dtype):
     cfg, change = FAR[what]
-    n = 90 if backend == "cpu" else 400
+    n = 90 if backend == "cpu" else 420
     folder = folders(f"far_{what}", dtype, cfg, 9, change)
     ordinary = [t if t != MARKER else MARKER + 1 for t in seqs_for(cfg, [n], seed=40)[0]]
     if what == "attention":
@@ -442,9 +442,10 @@ def test_far_tokens_count(backend, folders, what, dtype):
                 continue          # (the host backend is slow)
             r = runner_for(folder, dtype, backend, U.max_live_tokens(steps))
             # (these weights are large on purpose, and so are the rounding errors: 32-bit sums, and bfloat16 scores under a
-            # high temperature; losing the marker moves the last rows by 0.4 of their spread and more)
+            # high temperature, gates that open steeply: a single row may be off by more than elsewhere, but no more than one in
+            # fifty by more than the bound; losing the marker moves every row behind it)
             assert_rows(U.replay(r, steps)["r0"], want, dtype, f"far {what} {dtype} {kind}, the marker at {at}",
-                        1e-4 if dtype == "float32" else 0.15 if what == "attention" else None)
+                        1e-4 if dtype == "float32" else 0.15 if what == "attention" else None, worst=0.3)
 
 
 def test_chunk_edges_in_prompts_and_in_decoding(backend, folders):
