@@ -21,6 +21,10 @@ decode steps and prefill (`fp32`).  Peaks are the published ones of MI355X.
     python bench.py --only pafivik [--width 1024] [--kernel-times]   four Pafivik layers (lightning, channel_delta, attention,
                                                              channel_delta, each with sixteen experts and a shared one) beside
                                                              four Ridopel layers of the same width: prefill and decode
+    python bench.py --only dogalorn [--width 1024] [--kernel-times]  four Dogalorn layers (attention in chunks beside a minGRU,
+                                                             Mamba2, Mamba2, the pair again; dense feed-forwards; the stream in two
+                                                             copies) beside four Pafivik layers with dense feed-forwards of the same
+                                                             width (attention, lightning, lightning, attention): prefill and decode
 """
 import argparse
 import json
@@ -190,8 +194,8 @@ def main():
     ap.add_argument("--shape", choices=["xl", "large", "medium"], default=None,
                     help="--only decode / prefill / replay: the layer sizes of BASELINE.json's configs[2], [3] or [4] "
                          "(default xl; for replay medium)")
-    ap.add_argument("--width", type=int, default=0, help="--only ridopel, --only pafivik: one width instead of 1,024 and 2,048")
-    ap.add_argument("--only", choices=["decode", "prefill", "serving", "replay", "ridopel", "pafivik"], default=None,
+    ap.add_argument("--width", type=int, default=0, help="--only ridopel, pafivik, dogalorn: one width instead of 1,024 and 2,048")
+    ap.add_argument("--only", choices=["decode", "prefill", "serving", "replay", "ridopel", "pafivik", "dogalorn"], default=None,
                     help="run one workload and print a short line (decode, prefill: for profiling; serving: "
                          "BASELINE.json's configs[3], GPT-2 Large shape, 64 requests through the scheduler; replay: "
                          "configs[4], GPT-2 Medium shape, against the plain implementation)")
@@ -205,6 +209,8 @@ def main():
         return ridopel(a)
     if a.only == "pafivik":
         return pafivik(a)
+    if a.only == "dogalorn":
+        return dogalorn(a)
     if a.only == "replay":
         a.shape = a.shape or "medium"      # (configs[4] as written; --shape xl: the same replay at configs[2]'s sizes)
         return replay(a)
@@ -300,6 +306,40 @@ def pafivik_configs(width, layers=4, vocab=32000, positions=2048):
     paf = dict(architecture="Pafivik", vocab=vocab, width=width, norm=dict(eps=1e-5), embedding=dict(scale=1.0), residual_mult=0.5,
                layers=[kinds[i % 4] for i in range(layers)], max_positions=positions, n_positions=positions, vocab_size=vocab)
     return paf, ridopel_configs(width, layers, vocab, positions)[0]
+
+
+def dogalorn_configs(width, layers=4, vocab=32000, positions=2048):
+    """-> (a Dogalorn config, a Pafivik config) of the same width, layers, vocabulary and positions, both with dense
+    feed-forwards four times the width.  The Dogalorn layers: attention in chunks of 512 (heads of 64, a key head for every
+    four, a table of 32 distance biases) beside a minGRU of the model's width; Mamba2 (heads of 64 values, twice the width in
+    all, states of 128, four taps); Mamba2; the pair again; the stream in two copies; token rows plus rows picked by pairs.
+    The Pafivik layers: attention (heads of 64, a key head for every four), lightning (heads of 64 keys x 128 values), lightning,
+    attention."""
+    H = width // 64
+    ff = dict(kind="dense", ff=4 * width)
+    par = dict(type="parallel", mlp=ff, mixer=dict(
+        left=dict(heads=H, kv_heads=max(1, H // 4), dim=64, vdim=64, scale=0.125, bias_max=400, mask=dict(size=512), bias_buckets=32),
+        right=dict(width=width)))
+    mam = dict(type="mamba2", mlp=ff, mixer=dict(heads=2 * H, vdim=64, state=128, groups=1, conv=4, norm_groups=1))
+    kinds = [par, mam, mam, par]
+    dog = dict(architecture="Dogalorn", vocab=vocab, width=width, norm=dict(eps=1e-5), streams=2, logit_scale=1.0,
+               embedding=dict(bigram=dict(buckets=100003, mul_prev=31, mul_cur=17)), layers=[kinds[i % 4] for i in range(layers)],
+               max_positions=positions, n_positions=positions, vocab_size=vocab)
+    Hl = width // 128
+    att = dict(type="attention", mlp=ff, mixer=dict(heads=H, kv_heads=max(1, H // 4), dim=64, vdim=64, scale=0.125,
+                                                    rot=dict(base=10000.0, dims=64)))
+    lig = dict(type="lightning", mlp=ff, mixer=dict(heads=Hl, dim=64, vdim=128, decay=[1.0 - 2.0 ** -(5 + 3 * h / Hl) for h in range(Hl)]))
+    kinds = [att, lig, lig, att]
+    paf = dict(architecture="Pafivik", vocab=vocab, width=width, norm=dict(eps=1e-5), embedding=dict(scale=1.0), residual_mult=0.5,
+               layers=[kinds[i % 4] for i in range(layers)], max_positions=positions, n_positions=positions, vocab_size=vocab)
+    return dog, paf
+
+
+def dogalorn(a):
+    """Prefill and decode steps of four Dogalorn layers beside four Pafivik layers of the same width with the same dense
+    feed-forwards (the closest of the framework's models: an attention over pages, recurrences with a matrix state, norms
+    without a mean); with --kernel-times each model's kernels."""
+    return side_by_side(a, ("dogalorn", "pafivik"), dogalorn_configs)
 
 
 def pafivik(a):

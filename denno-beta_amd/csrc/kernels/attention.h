@@ -57,6 +57,13 @@ int dn_attention_flash(const void* q, int ldq, void* out, int ldo, const void* k
                        const int32_t* tile_row0, const int32_t* tile_nrows, const int32_t* tile_pos0, int n_tiles,
                        int H, int Hkv, int dh, int page_size, float scale, int window, hipStream_t stream);
 
+// dn_attention_flash with chunks, a bias by distance and a sink (ScoreExtras); with any of them, pages of a power of two
+int dn_attention_flash_extras(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
+                              const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,
+                              const int32_t* tile_row0, const int32_t* tile_nrows, const int32_t* tile_pos0, int n_tiles,
+                              int H, int Hkv, int dh, int page_size, float scale, int window, int chunk, const float* bias,
+                              int span, int sink, hipStream_t stream);
+
 // bfloat16, one row per request (tile s = request s = row s); the context is cut into n_splits runs of
 // `chunks` chunks of waves * 64 keys; part: device memory for n_tiles * H * n_splits * (dh + 2) floats
 // of split results (not touched when n_splits == 1).  tile_row0 is not read: tile s is row s of q and
@@ -68,6 +75,13 @@ int dn_attention_decode(const void* q, int ldq, void* out, int ldo, const void* 
                         const int32_t* tile_row0, const int32_t* tile_pos0, int n_tiles, float* part, int n_splits,
                         int chunks, int waves, int H, int Hkv, int dh, int page_size, float scale, int window,
                         hipStream_t stream);
+
+// dn_attention_decode with chunks, a bias by distance and a sink (ScoreExtras); with any of them, pages of a power of two
+int dn_attention_decode_extras(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
+                               const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,
+                               const int32_t* tile_row0, const int32_t* tile_pos0, int n_tiles, float* part, int n_splits,
+                               int chunks, int waves, int H, int Hkv, int dh, int page_size, float scale, int window,
+                               int chunk, const float* bias, int span, int sink, hipStream_t stream);
 
 // dn_attention_decode for callers that cannot allocate device memory (code under HIP graph capture,
 // tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.

@@ -621,15 +621,18 @@ typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
 // POW2: the page size is a power of two (page_size = 1 << page_shift), so that a key's page and its place in
 // the page are a shift and a mask: a tile's keys need four such pairs a step, and a division by a number
 // known only at run time is some twenty-five vector instructions.
-template <int DH16, int GROUPS, int TPS, bool POW2>     // head size / 16; groups of 4 waves; tiles a wave takes per step
+// EXTRAS: chunks, a bias by distance and a sink (ScoreExtras).  A score is then the scaled product plus the bias, both
+// in units of log2(e), made before the maximum is taken (the largest product is no longer the largest score).
+template <int DH16, int GROUPS, int TPS, bool POW2, bool EXTRAS = false>     // head size / 16; groups of 4 waves; tiles a wave takes per step
 __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(DH16 > 12 && GROUPS == 1 ? 1 : 2))) void kernel(
     const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_row0,
     const int32_t* __restrict__ tile_nrows, const int32_t* __restrict__ tile_pos0, int H, int Hkv, int page_size,
-    int page_shift, float scale, int window) {
+    int page_shift, float scale, int window, ScoreExtras ex) {
   constexpr int DH = DH16 * 16;
   constexpr int DB = (DH + 31) / 32;
+  const int chunk = EXTRAS ? ex.chunk : 0;
   auto page_index = [&](int key) { return POW2 ? key >> page_shift : key / page_size; };
   auto page_offset = [&](int key) { return POW2 ? key & (page_size - 1) : key % page_size; };
   constexpr int CH = DH / 8;                 // 16-byte chunks in a key
@@ -663,11 +666,13 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(DH
   const bool row_ok = wrow0 + qcol < nrows;
   const int my_row = min(wrow0 + qcol, nrows - 1);
   const int my_pos = pos0 + my_row;
-  const int my_lo = window > 0 ? max(0, my_pos - window + 1) : 0;
-  const int lo_w = window > 0 ? max(0, pos0 + wrow0 - window + 1) : 0;      // this wave's keys
+  const int my_lo = first_key(my_pos, window, chunk);
+  const int lo_w = first_key(pos0 + wrow0, window, chunk);      // this wave's keys
   const int hi_w = pos0 + min(wrow0 + 31, nrows - 1);
-  const int lo_g = window > 0 ? max(0, pos0 - window + 1) : 0;              // the workgroup's
+  const int lo_last = first_key(hi_w, window, chunk);           // the first key of the wave's last row
+  const int lo_g = first_key(pos0, window, chunk);              // the workgroup's
   const int hi_g = pos0 + nrows - 1;
+  const float* bias = EXTRAS && ex.bias ? ex.bias + static_cast<size_t>(h) * ex.span : nullptr;
   const float NEG_INF = -INFINITY;
   const float scale2 = scale * 1.44269504088896340736f;    // log2(e)
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
@@ -797,9 +802,19 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(DH
 #pragma unroll
       for (int c = 0; c < TPS; ++c) {
         const int kw = kw0 + 32 * c;
-        const bool edge = kw + 31 > pos0 + wrow0 || (window > 0 && kw < hi_w - window + 1);
+        const bool edge = kw + 31 > pos0 + wrow0 || kw < lo_last;
         if (!act[c]) continue;
-        if (edge) {
+        if constexpr (EXTRAS) {
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int key = kw + 8 * (i / 4) + 4 * g + (i % 4);
+            const bool ok = key >= my_lo && key <= my_pos;
+            float sc = s[c][i] * scale2;
+            if (bias) sc = fmaf(bias[min(max(my_pos - key, 0), ex.span - 1)], 1.44269504088896340736f, sc);
+            s[c][i] = (!edge || ok) ? sc : NEG_INF;
+            tmax = fmaxf(tmax, s[c][i]);
+          }
+        } else if (edge) {
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
             int key = kw + 8 * (i / 4) + 4 * g + (i % 4);
@@ -812,7 +827,7 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(DH
           for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, s[c][i]);
         }
       }
-      tmax = fmaxf(tmax, other_half(tmax)) * scale2;      // (-inf stays -inf)
+      tmax = fmaxf(tmax, other_half(tmax)) * (EXTRAS ? 1.0f : scale2);      // (-inf stays -inf)
       float p[TPS][16];
       float psum = 0.f, alpha = 1.f;
       if (tmax > NEG_INF) {
@@ -822,7 +837,7 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(DH
         for (int c = 0; c < TPS; ++c)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
-            p[c][i] = __builtin_amdgcn_exp2f(fmaf(s[c][i], scale2, -m_new));  // a masked score is -inf: 0
+            p[c][i] = __builtin_amdgcn_exp2f(EXTRAS ? s[c][i] - m_new : fmaf(s[c][i], scale2, -m_new));  // a masked score is -inf: 0
             psum += p[c][i];
           }
         m = m_new;
@@ -887,12 +902,14 @@ __global__ __launch_bounds__(256 * GROUPS) __attribute__((amdgpu_waves_per_eu(DH
     const float f0 = m > NEG_INF ? __builtin_amdgcn_exp2f(m - m_new) : 0.f;
     const float f1 = m1 > NEG_INF ? __builtin_amdgcn_exp2f(m1 - m_new) : 0.f;
     l = l * f0 + l1 * f1;
+    m = m_new;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int i = 0; i < 16; ++i) o[db][i] = o[db][i] * f0 + join[2 + 16 * db + i] * f1;
   }
   if (has_rows && row_ok) {
+    if (EXTRAS && ex.sink) l += __builtin_amdgcn_exp2f(-m);      // (a key with score 0 and no value)
     const float inv = 1.0f / l;
     // rows, or packed rows (ldo == 0): four dims from a multiple of 4 are 8 bytes side by side in both
     const int orow_i = row0 + my_row;
@@ -918,7 +935,20 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
                                   const int32_t* tile_row0, const int32_t* tile_nrows, const int32_t* tile_pos0,
                                   int n_tiles, int H, int Hkv, int dh, int page_size, float scale, int window,
                                   hipStream_t stream) {
+  return dn_attention_flash_extras(q, ldq, out, ldo, k_pool, v_pool, block_tables, max_blocks, tile_seq, tile_row0, tile_nrows,
+                                   tile_pos0, n_tiles, H, Hkv, dh, page_size, scale, window, 0, nullptr, 0, 0, stream);
+}
+
+// With chunks, a bias by distance or a sink: pages of a power of two only.
+extern "C" int dn_attention_flash_extras(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
+                                         const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,
+                                         const int32_t* tile_row0, const int32_t* tile_nrows, const int32_t* tile_pos0,
+                                         int n_tiles, int H, int Hkv, int dh, int page_size, float scale, int window, int chunk,
+                                         const float* bias, int span, int sink, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
+  const bool extras = chunk > 0 || bias != nullptr || sink != 0;
+  if (chunk < 0 || (bias && span < 1)) return DN_ERR_SHAPE;
+  const ScoreExtras ex{chunk, bias, span, sink};
   // ldo == 0: out is a packed matrix of H * dh columns (a multiple of 32); the kernel takes the largest score
   // for the largest product of a query and a key, so the scale is positive
   if (!(scale > 0.f)) return DN_ERR_SHAPE;
@@ -935,16 +965,19 @@ extern "C" int dn_attention_flash(const void* q, int ldq, void* out, int ldo, co
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
   const bool pow2 = (1 << page_shift) == page_size;
-#define DN_FLASH_P(D, G, T, P)                                                                                        \
-  hipLaunchKernelGGL((flash::kernel<D, G, T, P>), grid, dim3(256 * G), 0, stream, static_cast<const bf16_t*>(q), ldq, \
+  if (extras && !pow2) return DN_ERR_SHAPE;
+#define DN_FLASH_P(D, G, T, P, X)                                                                                        \
+  hipLaunchKernelGGL((flash::kernel<D, G, T, P, X>), grid, dim3(256 * G), 0, stream, static_cast<const bf16_t*>(q), ldq, \
                      static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(k_pool),                             \
                      static_cast<const bf16_t*>(v_pool), block_tables, max_blocks, tile_seq, tile_row0, tile_nrows,   \
-                     tile_pos0, H, Hkv, page_size, page_shift, scale, window)
-#define DN_FLASH_G(D, G, T)    \
-  if (pow2)                    \
-    DN_FLASH_P(D, G, T, true); \
-  else                         \
-    DN_FLASH_P(D, G, T, false)
+                     tile_pos0, H, Hkv, page_size, page_shift, scale, window, ex)
+#define DN_FLASH_G(D, G, T)           \
+  if (extras)                         \
+    DN_FLASH_P(D, G, T, true, true);  \
+  else if (pow2)                      \
+    DN_FLASH_P(D, G, T, true, false); \
+  else                                \
+    DN_FLASH_P(D, G, T, false, false)
 #define DN_FLASH2(D) DN_FLASH_G(D, 2, 1)                      /* two groups of waves, a tile each */
 #define DN_FLASH1(D) DN_FLASH_G(D, 1, (D <= 6 ? 2 : 1))       /* one group, two tiles a step where registers allow */
   switch (dh) {
@@ -995,7 +1028,7 @@ namespace decode {
 // that is no power of two (48, 80, 96, ...) the lanes beyond the key's last piece hold zeros.
 constexpr int lanes_per_key(int dh) { return dh <= 16 ? 2 : dh <= 32 ? 4 : dh <= 64 ? 8 : dh <= 128 ? 16 : 32; }
 
-template <int DH, int WAVES, bool POW2>   // head size (a multiple of 16 up to 256); waves per workgroup
+template <int DH, int WAVES, bool POW2, bool EXTRAS = false>   // head size (a multiple of 16 up to 256); waves per workgroup; ScoreExtras
 __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out,
                                                        int ldo, const bf16_t* __restrict__ k_pool,
                                                        const bf16_t* __restrict__ v_pool,
@@ -1005,7 +1038,7 @@ __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __res
                                                        const int32_t* __restrict__ tile_pos0,
                                                        float* __restrict__ part, int n_splits, int chunks, int H,
                                                        int Hkv, int page_size, int page_shift, float scale,
-                                                       int window) {
+                                                       int window, ScoreExtras ex) {
   static_assert(DH % 16 == 0 && DH >= 16 && DH <= 256, "head size");
   constexpr int LPK = lanes_per_key(DH);
   constexpr int PIECES = DH / 8;         // 16-byte pieces of a key: the lanes sub < PIECES of its LPK
@@ -1029,7 +1062,8 @@ __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __res
   if (holds) qv = *reinterpret_cast<const bf16x8*>(q + static_cast<size_t>(row) * ldq + h * DH + sub * 8);
   if (tile_seq[tile] < 0) return;
   const int pos = tile_pos0[tile];
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int lo = first_key(pos, window, EXTRAS ? ex.chunk : 0);
+  const float* bias = EXTRAS && ex.bias ? ex.bias + static_cast<size_t>(h) * ex.span : nullptr;
   const int key0 = split * chunks * CHUNK;
   const float NEG_INF = -INFINITY;
   float* mypart = part + ((static_cast<size_t>(tile) * H + h) * n_splits + split) * (DH + 2);
@@ -1094,6 +1128,7 @@ __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __res
 #pragma unroll
         for (int i = 0; i < 8; ++i) dot = fmaf(qr[i], static_cast<float>(kv[u][i]), dot);
         dot = group_reduce<LPK>(dot, SumOp());
+        if (EXTRAS && bias) dot += bias[min(max(pos - key, 0), ex.span - 1)];
         sc[it0 + u] = (key >= lo && key <= pos) ? dot : NEG_INF;
       }
     }
@@ -1151,6 +1186,7 @@ __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __res
       }
     }
     if (n_splits == 1) {
+      if (EXTRAS && ex.sink) L += __expf(-M);      // (a key with score 0 and no value)
       out[ldo > 0 ? static_cast<size_t>(row) * ldo + h * DH + d : packed_index(row, h * DH + d, H * DH / 32)] =
           from_float<bf16_t>(A / L);
     } else {
@@ -1165,7 +1201,7 @@ __global__ __launch_bounds__(WAVES * 64) void partial_kernel(const bf16_t* __res
 
 __global__ void join_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, int ldo,
                             const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_row0, int n_splits,
-                            int H, int DH) {
+                            int H, int DH, int sink) {
   const int tile = blockIdx.x, h = blockIdx.y;
   if (tile_seq[tile] < 0) return;
   const float* base = part + (static_cast<size_t>(tile) * H + h) * n_splits * (DH + 2);
@@ -1181,6 +1217,7 @@ __global__ void join_kernel(const float* __restrict__ part, bf16_t* __restrict__
         A += ps[2 + d] * f;
       }
     }
+    if (sink) L += __expf(-M);
     out[ldo > 0 ? static_cast<size_t>(tile) * ldo + h * DH + d : packed_index(tile, h * DH + d, H * DH / 32)] =
         from_float<bf16_t>(A / L);
   }
@@ -1196,7 +1233,22 @@ extern "C" int dn_attention_decode(const void* q, int ldq, void* out, int ldo, c
                                    const int32_t* tile_row0, const int32_t* tile_pos0, int n_tiles, float* part,
                                    int n_splits, int chunks, int waves, int H, int Hkv, int dh, int page_size,
                                    float scale, int window, hipStream_t stream) {
+  return dn_attention_decode_extras(q, ldq, out, ldo, k_pool, v_pool, block_tables, max_blocks, tile_seq, tile_row0, tile_pos0,
+                                    n_tiles, part, n_splits, chunks, waves, H, Hkv, dh, page_size, scale, window, 0, nullptr, 0, 0,
+                                    stream);
+}
+
+// With chunks, a bias by distance or a sink: pages of a power of two only.
+extern "C" int dn_attention_decode_extras(const void* q, int ldq, void* out, int ldo, const void* k_pool, const void* v_pool,
+                                          const int32_t* block_tables, int max_blocks, const int32_t* tile_seq,
+                                          const int32_t* tile_row0, const int32_t* tile_pos0, int n_tiles, float* part,
+                                          int n_splits, int chunks, int waves, int H, int Hkv, int dh, int page_size,
+                                          float scale, int window, int chunk, const float* bias, int span, int sink,
+                                          hipStream_t stream) {
   if (n_tiles <= 0) return 0;
+  const bool extras = chunk > 0 || bias != nullptr || sink != 0;
+  if (chunk < 0 || (bias && span < 1)) return DN_ERR_SHAPE;
+  const ScoreExtras ex{chunk, bias, span, sink};
   if (Hkv < 1 || H % Hkv != 0 || page_size % 16 != 0 || max_blocks < 1 || n_splits < 1 || chunks < 1 ||
       ldq % 8 != 0 || ldo < 0 || (ldo == 0 && (H * dh) % 32 != 0) || reinterpret_cast<uintptr_t>(q) % 16 != 0 || reinterpret_cast<uintptr_t>(k_pool) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(v_pool) % 16 != 0)
@@ -1206,17 +1258,20 @@ extern "C" int dn_attention_decode(const void* q, int ldq, void* out, int ldo, c
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
   const bool pow2 = (1 << page_shift) == page_size;
-#define DN_DECODE_P(L, W, P)                                                                                          \
-  hipLaunchKernelGGL((decode::partial_kernel<L, W, P>), grid, block, 0, stream, static_cast<const bf16_t*>(q), ldq,   \
+  if (extras && !pow2) return DN_ERR_SHAPE;
+#define DN_DECODE_P(L, W, P, X)                                                                                       \
+  hipLaunchKernelGGL((decode::partial_kernel<L, W, P, X>), grid, block, 0, stream, static_cast<const bf16_t*>(q), ldq, \
                      static_cast<bf16_t*>(out), ldo, static_cast<const bf16_t*>(k_pool),                              \
                      static_cast<const bf16_t*>(v_pool), block_tables, max_blocks, tile_seq, tile_row0, tile_pos0,    \
-                     part, n_splits, chunks, H, Hkv, page_size, page_shift, scale, window)
+                     part, n_splits, chunks, H, Hkv, page_size, page_shift, scale, window, ex)
 #define DN_DECODE_W(L, W)    \
   do {                       \
-    if (pow2)                \
-      DN_DECODE_P(L, W, true);  \
+    if (extras)              \
+      DN_DECODE_P(L, W, true, true);   \
+    else if (pow2)           \
+      DN_DECODE_P(L, W, true, false);  \
     else                     \
-      DN_DECODE_P(L, W, false); \
+      DN_DECODE_P(L, W, false, false); \
   } while (0)
 #define DN_DECODE(D)                  \
   if (waves == 16) {                  \
@@ -1249,7 +1304,7 @@ extern "C" int dn_attention_decode(const void* q, int ldq, void* out, int ldo, c
 #undef DN_DECODE_P
   if (n_splits > 1)
     hipLaunchKernelGGL(decode::join_kernel, dim3(n_tiles, H), dim3(64), 0, stream, part, static_cast<bf16_t*>(out),
-                       ldo, tile_seq, tile_row0, n_splits, H, dh);
+                       ldo, tile_seq, tile_row0, n_splits, H, dh, sink);
   return dn_launch_status();
 }
 

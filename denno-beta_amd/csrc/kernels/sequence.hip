@@ -124,13 +124,15 @@ __global__ __launch_bounds__(256) void conv_rows_kernel(const float* h, size_t l
   const int t = blockIdx.x;
   const int s = request_of(row_start, S, t);
   const int slot = slots[s];
+  // (a row's channels are shared out among the workgroups of the grid's second dimension, 256 at a time)
+  const int c0 = blockIdx.y * 256 + threadIdx.x, cstep = gridDim.y * 256;
   if (slot < 0 || t >= row_start[S]) {      // a padding row: zeros, so that what follows works on numbers
-    for (int c = threadIdx.x; c < width; c += 256) store_as(out, static_cast<size_t>(t) * ldo + c, out_dt, 0.f);
+    for (int c = c0; c < width; c += cstep) store_as(out, static_cast<size_t>(t) * ldo + c, out_dt, 0.f);
     return;
   }
   const int i = t - row_start[s];
   const float* past = hist + static_cast<size_t>(slot) * hist_stride;
-  for (int c = threadIdx.x; c < width; c += 256) {
+  for (int c = c0; c < width; c += cstep) {
     float acc = (identity ? h[static_cast<size_t>(t) * ldh + c] : 0.f) + (bias ? bias[c] : 0.f);
     for (int j = 0; j < taps; ++j) {
       const int src = i - taps + 1 + j;
@@ -610,47 +612,106 @@ __global__ __launch_bounds__(256) void step_sizes_kernel(const float* z, size_t 
 
 // ---- a recurrence of single numbers whose gates read the token alone ----------------------------------------------
 // z = sigmoid(a[t, c] + bias_a[c]); u = b[t, c] + bias_b[c]; cand = u >= 0 ? u + 1/2 : sigmoid(u); S <- (1 - z) S + z cand;
-// out[t, c] = S * silu(g[t, c]).  A thread owns a channel of a request and walks its rows in order; eight rows' numbers are
-// asked for at a time, the next eight before the current ones are worked on.  A row's result depends on the rows before it
-// alone, in one order.
-__global__ __launch_bounds__(64) void gate_scan_kernel(const float* a, size_t lda, const float* b, size_t ldb, const float* g, size_t ldg,
-                                                       const float* bias_a, const float* bias_b, float* state, size_t slot_stride,
-                                                       const int* row_start, const int* slots, int width, void* out, int out_dt,
-                                                       size_t ldo) {
+// out[t, c] = S * silu(g[t, c]).  A workgroup owns 64 channels of a request, a lane a channel.  Its WAVES waves take
+// eight rows each of every run of 8 WAVES rows: a wave first walks its rows from a state of zero, which gives the
+// product P of its (1 - z) and what it adds, Q, so that the state behind its rows is P S + Q for any state S before
+// them; the waves' (P, Q) meet in LDS, every wave folds those of the waves before it into the state at the run's
+// start, in order, and walks its rows again from there.  A step of single rows takes one wave, which walks them once.
+// A row's result depends on the rows before it alone; how the rows were cut changes it by rounding only.
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gate_scan_kernel(const float* a, size_t lda, const float* b, size_t ldb, const float* g,
+                                                               size_t ldg, const float* bias_a, const float* bias_b, float* state,
+                                                               size_t slot_stride, const int* row_start, const int* slots, int width,
+                                                               void* out, int out_dt, size_t ldo) {
   constexpr int TB = 8;
-  const int s = blockIdx.y, c = blockIdx.x * 64 + threadIdx.x;
+  __shared__ float shp[2][WAVES][64], shq[2][WAVES][64];
+  const int s = blockIdx.y, lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+  const int c = blockIdx.x * 64 + lane;
   const int slot = slots[s];
-  if (slot < 0 || c >= width) return;
+  if (slot < 0) return;      // (the whole workgroup)
   const int row0 = row_start[s], row1 = row_start[s + 1];
   if (row0 >= row1) return;
-  const float ba = bias_a ? bias_a[c] : 0.f, bb = bias_b ? bias_b[c] : 0.f;
-  float* sp = state + static_cast<size_t>(slot) * slot_stride + c;
-  float S = *sp;
+  const bool live = c < width;
+  const int cc = live ? c : width - 1;
+  const float ba = bias_a ? bias_a[cc] : 0.f, bb = bias_b ? bias_b[cc] : 0.f;
+  float* sp = state + static_cast<size_t>(slot) * slot_stride + cc;
+  float S0 = *sp;      // the state before the run that is worked on; every wave keeps it
   float na[TB], nb[TB], ng[TB];
   auto fetch = [&](int t0) {
 #pragma unroll
     for (int i = 0; i < TB; ++i) {
       const size_t t = min(t0 + i, row1 - 1);
-      na[i] = a[t * lda + c], nb[i] = b[t * ldb + c], ng[i] = g[t * ldg + c];
+      na[i] = a[t * lda + cc], nb[i] = b[t * ldb + cc], ng[i] = g[t * ldg + cc];
     }
   };
-  fetch(row0);
-  for (int t0 = row0; t0 < row1; t0 += TB) {
-    float ca[TB], cb[TB], cg[TB];
-#pragma unroll
-    for (int i = 0; i < TB; ++i) ca[i] = na[i], cb[i] = nb[i], cg[i] = ng[i];
-    if (t0 + TB < row1) fetch(t0 + TB);
+  fetch(row0 + wave * TB);
+  int par = 0;
+  for (int t0 = row0; t0 < row1; t0 += WAVES * TB, par ^= 1) {
+    const int mine = t0 + wave * TB;
+    float keep[TB], add[TB], gate[TB];
+    float P = 1.f, Q = 0.f;
 #pragma unroll
     for (int i = 0; i < TB; ++i) {
-      if (t0 + i < row1) {
-        const float z = sigmoid_f(ca[i] + ba), u = cb[i] + bb;
-        const float cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
-        S = fmaf(z, cand - S, S);
-        store_as(out, static_cast<size_t>(t0 + i) * ldo + c, out_dt, S * activation(ACT_SILU, cg[i], 0.f));
-      }
+      const float z = sigmoid_f(na[i] + ba), u = nb[i] + bb;
+      const float cand = u >= 0.f ? u + 0.5f : sigmoid_f(u);
+      const bool row = mine + i < row1;
+      keep[i] = row ? 1.0f - z : 1.0f;      // (places beyond the last row change nothing)
+      add[i] = row ? z * cand : 0.f;
+      gate[i] = ng[i];
+      P *= keep[i];
+      Q = fmaf(keep[i], Q, add[i]);
     }
+    if (t0 + WAVES * TB < row1) fetch(mine + WAVES * TB);
+    float S = S0;
+    if constexpr (WAVES > 1) {
+      shp[par][wave][lane] = P, shq[par][wave][lane] = Q;
+      __syncthreads();      // (the other half of LDS is what the run before used: one barrier a run)
+      float run = S0;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) {
+        if (w == wave) S = run;
+        run = fmaf(shp[par][w][lane], run, shq[par][w][lane]);
+      }
+      S0 = run;
+    }
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      S = fmaf(keep[i], S, add[i]);
+      if (live && mine + i < row1)
+        store_as(out, static_cast<size_t>(mine + i) * ldo + c, out_dt, S * activation(ACT_SILU, gate[i], 0.f));
+    }
+    if constexpr (WAVES == 1) S0 = S;
   }
-  *sp = S;
+  if (live && wave == 0) *sp = S0;
+}
+
+// ---- queries and keys normed as whole vectors, keys and values to the cache -----------------------------------------
+// A row of z is [q: qw | k: kw].  q_out[t] = q / rms(q) * wq; the key that goes to the cache is k / rms(k) * wk, the value
+// k as it is (pools [page][key head][offset][dim] and [page][key head][dim][offset], the row's place from slot_map; a
+// negative place: nothing is written).  One workgroup a row, the sums as in rmsnorm_kernel.
+__global__ __launch_bounds__(256) void norm_pair_write_kernel(const float* z, size_t ldz, int qw, int kw, const float* wq, const float* wk,
+                                                              float eps, void* q_out, size_t ldq, const int* slot_map, void* k_pool,
+                                                              void* v_pool, int dh, int page_size, int dt, int write) {
+  __shared__ float sh[4];
+  const size_t t = blockIdx.x;
+  const float* row = z + t * ldz;
+  float sq = 0.f, sk = 0.f;
+  for (int c = threadIdx.x; c < qw; c += 256) sq = fmaf(row[c], row[c], sq);
+  for (int c = threadIdx.x; c < kw; c += 256) sk = fmaf(row[qw + c], row[qw + c], sk);
+  sq = block_sum_256(sq, sh);
+  sk = block_sum_256(sk, sh);
+  const float iq = 1.0f / sqrtf(sq / static_cast<float>(qw) + eps), ik = 1.0f / sqrtf(sk / static_cast<float>(kw) + eps);
+  for (int c = threadIdx.x; c < qw; c += 256) store_as(q_out, t * ldq + c, dt, row[c] * iq * wq[c]);
+  const int slot = slot_map[t];
+  if (!write || slot < 0) return;
+  const int page = slot / page_size, off = slot % page_size, Hkv = kw / dh;
+  for (int c = threadIdx.x; c < kw; c += 256) {
+    const int h = c / dh, d = c % dh;
+    const size_t base = (static_cast<size_t>(page) * Hkv + h) * page_size * dh;
+    const float k = row[qw + c];
+    store_as(k_pool, base + static_cast<size_t>(off) * dh + d, dt, k * ik * wk[c]);
+    store_as(v_pool, base + static_cast<size_t>(d) * page_size + off, dt, k);
+  }
 }
 
 // ---- several copies of the stream -----------------------------------------------------------------------------------
@@ -693,9 +754,12 @@ __global__ __launch_bounds__(256) void streams_read_kernel(const float* xs, size
 
 // write: every copy anew from the old ones and a sublayer's result y: x_t <- sum_s mix[s][t] x_s + w_out[t] * y (s ascending).
 // next_in given: the same workgroup then reads the new copies for the next sublayer, as streams_read_kernel does, into `out`.
+// y2 given: the result is the mean of two branches, each normed over the width first with a weight of its own:
+// y = (y / rms(y) * by + y2 / rms(y2) * by2) / 2 (the sums as rmsnorm_add_kernel makes them, one branch after the other).
 __global__ __launch_bounds__(256) void streams_write_kernel(float* xs, size_t plane, int n, const float* mix, const float* w_out, const float* y,
-                                                            size_t ldy, const float* next_in, const float* g, float eps, void* out, int out_dt,
-                                                            size_t ldo, int width) {
+                                                            size_t ldy, const float* y2, size_t ldy2, const float* by, const float* by2,
+                                                            float beps, const float* next_in, const float* g, float eps, void* out,
+                                                            int out_dt, size_t ldo, int width) {
   __shared__ float sh[4];
   __shared__ float sm[STREAMS_MAX * STREAMS_MAX + 2 * STREAMS_MAX];
   const size_t row = blockIdx.x;
@@ -707,12 +771,24 @@ __global__ __launch_bounds__(256) void streams_write_kernel(float* xs, size_t pl
   __syncthreads();
   const float* wo = sm + STREAMS_MAX * STREAMS_MAX;
   const float* wn = wo + STREAMS_MAX;
+  float inv1 = 0.f, inv2 = 0.f;
+  if (y2) {
+    float s1 = 0.f, s2 = 0.f;
+    for (int c = threadIdx.x; c < width; c += 256) {
+      const float a = y[row * ldy + c], b = y2[row * ldy2 + c];
+      s1 = fmaf(a, a, s1), s2 = fmaf(b, b, s2);
+    }
+    s1 = block_sum_256(s1, sh);
+    s2 = block_sum_256(s2, sh);
+    inv1 = 1.0f / sqrtf(s1 / static_cast<float>(width) + beps), inv2 = 1.0f / sqrtf(s2 / static_cast<float>(width) + beps);
+  }
   float ss = 0.f;
   for (int c = threadIdx.x; c < width; c += 256) {
     float old[STREAMS_MAX];
 #pragma unroll
     for (int s = 0; s < STREAMS_MAX; ++s) old[s] = s < n ? xs[s * plane + row * width + c] : 0.f;
-    const float yc = y[row * ldy + c];
+    float yc = y[row * ldy + c];
+    if (y2) yc = fmaf(0.5f, y2[row * ldy2 + c] * inv2 * by2[c], fmaf(0.5f, yc * inv1 * by[c], 0.f));
     float u = 0.f;
 #pragma unroll
     for (int t = 0; t < STREAMS_MAX; ++t) {
@@ -799,7 +875,8 @@ int dn_conv_rows(const float* h, long long ldh, const float* w, const float* bia
   if (!float_kind(out_dt)) return DN_ERR_DTYPE;
   if (taps < 1 || S < 1 || ldh < width || ldo < width) return DN_ERR_SHAPE;
   if (T == 0) return 0;
-  hipLaunchKernelGGL(conv_rows_kernel, dim3(T), dim3(256), 0, stream, h, static_cast<size_t>(ldh), w, bias, hist, row_start, slots, S, width,
+  // (few rows: a workgroup for every 256 channels of a row, so that a step of decoded tokens is more than a handful of workgroups)
+  hipLaunchKernelGGL(conv_rows_kernel, dim3(T, T <= 256 ? (width + 255) / 256 : 1), dim3(256), 0, stream, h, static_cast<size_t>(ldh), w, bias, hist, row_start, slots, S, width,
                      taps, identity, silu, out, out_dt, static_cast<size_t>(ldo), static_cast<size_t>(hist_stride));
   return dn_launch_status();
 }
@@ -959,14 +1036,20 @@ int dn_step_sizes(const float* z, long long ldz, const float* bias, const float*
 }
 
 int dn_gate_scan(const float* a, long long lda, const float* b, long long ldb, const float* g, long long ldg, const float* bias_a,
-                 const float* bias_b, float* state, long long slot_stride, const int* row_start, const int* slots, int S, int width,
+                 const float* bias_b, float* state, long long slot_stride, const int* row_start, const int* slots, int S, int T, int width,
                  void* out, int out_dt, long long ldo, hipStream_t stream) {
   if (!float_kind(out_dt)) return DN_ERR_DTYPE;
   if (width < 1 || S > 65535) return DN_ERR_SHAPE;
   if (S == 0) return 0;
-  hipLaunchKernelGGL(gate_scan_kernel, dim3((width + 63) / 64, S), dim3(64), 0, stream, a, static_cast<size_t>(lda), b,
-                     static_cast<size_t>(ldb), g, static_cast<size_t>(ldg), bias_a, bias_b, state, static_cast<size_t>(slot_stride), row_start,
-                     slots, width, out, out_dt, static_cast<size_t>(ldo));
+  // (decoded tokens, a row or two a request: one wave; portions: sixteen waves of eight rows each at a time)
+  if (T <= 2 * S)
+    hipLaunchKernelGGL(gate_scan_kernel<1>, dim3((width + 63) / 64, S), dim3(64), 0, stream, a, static_cast<size_t>(lda), b,
+                       static_cast<size_t>(ldb), g, static_cast<size_t>(ldg), bias_a, bias_b, state, static_cast<size_t>(slot_stride),
+                       row_start, slots, width, out, out_dt, static_cast<size_t>(ldo));
+  else
+    hipLaunchKernelGGL(gate_scan_kernel<16>, dim3((width + 63) / 64, S), dim3(1024), 0, stream, a, static_cast<size_t>(lda), b,
+                       static_cast<size_t>(ldb), g, static_cast<size_t>(ldg), bias_a, bias_b, state, static_cast<size_t>(slot_stride),
+                       row_start, slots, width, out, out_dt, static_cast<size_t>(ldo));
   return dn_launch_status();
 }
 
@@ -981,13 +1064,25 @@ int dn_streams_read(const float* xs, long long plane, int n, const float* w_in, 
 }
 
 int dn_streams_write(float* xs, long long plane, int n, const float* mix, const float* w_out, const float* y, long long ldy,
-                     const float* next_in, const float* g, float eps, void* out, int out_dt, long long ldo, int T, int width,
-                     hipStream_t stream) {
+                     const float* y2, long long ldy2, const float* by, const float* by2, float beps, const float* next_in,
+                     const float* g, float eps, void* out, int out_dt, long long ldo, int T, int width, hipStream_t stream) {
   if (next_in && !float_kind(out_dt)) return DN_ERR_DTYPE;
-  if (n < 1 || n > STREAMS_MAX || width < 1 || (next_in && !out)) return DN_ERR_SHAPE;
+  if (n < 1 || n > STREAMS_MAX || width < 1 || (next_in && !out) || (y2 && (!by || !by2))) return DN_ERR_SHAPE;
   if (T == 0) return 0;
   hipLaunchKernelGGL(streams_write_kernel, dim3(T), dim3(256), 0, stream, xs, static_cast<size_t>(plane), n, mix, w_out, y,
-                     static_cast<size_t>(ldy), next_in, g, eps, out, out_dt, static_cast<size_t>(ldo), width);
+                     static_cast<size_t>(ldy), y2, static_cast<size_t>(ldy2), by, by2, beps, next_in, g, eps, out, out_dt,
+                     static_cast<size_t>(ldo), width);
+  return dn_launch_status();
+}
+
+int dn_norm_pair_write(const float* z, long long ldz, int qw, int kw, const float* wq, const float* wk, float eps, void* q_out,
+                       long long ldq, const int* slot_map, void* k_pool, void* v_pool, int T, int Hkv, int dh, int page_size,
+                       int dt, int write, hipStream_t stream) {
+  if (!float_kind(dt)) return DN_ERR_DTYPE;
+  if (qw < 1 || kw != Hkv * dh || page_size < 1 || ldz < qw + kw || ldq < qw) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(norm_pair_write_kernel, dim3(T), dim3(256), 0, stream, z, static_cast<size_t>(ldz), qw, kw, wq, wk, eps, q_out,
+                     static_cast<size_t>(ldq), slot_map, k_pool, v_pool, dh, page_size, dt, write);
   return dn_launch_status();
 }
 

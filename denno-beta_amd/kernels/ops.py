@@ -122,6 +122,8 @@ def _declare(name, lib):
             "dn_attention_rows_tile": [I],
             "dn_attention_extras": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, I, P, I, I, I, P],
             "dn_attention_rows_extras": [P, I, P, I, P, P, P, I, P, P, I, P, I, I, I, I, I, F, I, I, P, I, I, I, P],
+            "dn_attention_flash_extras": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, I, P, I, I, P],
+            "dn_attention_decode_extras": [P, I, P, I, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, I, F, I, I, P, I, I, P],
             "dn_attention_flash": [P, I, P, I, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, P],
             "dn_attention_decode": [P, I, P, I, P, P, P, I, P, P, P, I, P, I, I, I, I, I, I, I, F, I, P],
         },
@@ -143,9 +145,10 @@ def _declare(name, lib):
                               I, I, I, I, I, I, I, I, I, P, c_longlong, P],
             "dn_head_norm": [P, c_longlong, P, I, F, P, c_longlong, I, I, P, c_longlong, P, I, P, I, c_longlong, I, I, I, P],
             "dn_step_sizes": [P, c_longlong, P, P, P, c_longlong, I, I, I, P, c_longlong, P, c_longlong, P],
-            "dn_gate_scan": [P, c_longlong, P, c_longlong, P, c_longlong, P, P, P, c_longlong, P, P, I, I, P, I, c_longlong, P],
+            "dn_gate_scan": [P, c_longlong, P, c_longlong, P, c_longlong, P, P, P, c_longlong, P, P, I, I, I, P, I, c_longlong, P],
             "dn_streams_read": [P, c_longlong, I, P, P, F, P, I, c_longlong, P, I, I, P],
-            "dn_streams_write": [P, c_longlong, I, P, P, P, c_longlong, P, P, F, P, I, c_longlong, I, I, P],
+            "dn_streams_write": [P, c_longlong, I, P, P, P, c_longlong, P, c_longlong, P, P, F, P, P, F, P, I, c_longlong, I, I, P],
+            "dn_norm_pair_write": [P, c_longlong, I, I, P, P, F, P, c_longlong, P, P, P, I, I, I, I, I, I, P],
         },
         "grouped": {
             "dn_heads_linear": [P, I, c_longlong, I, I, P, I, P, I, c_longlong, I, I, I, I, I, I, P],
@@ -657,7 +660,9 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
     _need(chunk >= 0, "attention: chunk")
     lib = _lib("attention")
     # (the kernel for portions takes the largest score for the largest product: a scale that is not positive goes the plain way)
-    fast = q.dtype == torch.bfloat16 and ps % 16 == 0 and ldq % 8 == 0 and q.data_ptr() % 16 == 0 and scale > 0 and not extras
+    # (with chunks, a bias or a sink the two bfloat16 kernels take pages of a power of two)
+    fast = (q.dtype == torch.bfloat16 and ps % 16 == 0 and ldq % 8 == 0 and q.data_ptr() % 16 == 0 and scale > 0
+            and (not extras or ps & (ps - 1) == 0))
     decode = fast and decode_attention_applies(q.dtype, ps, dh, single_rows, max_context)
     _need(not out_packed or (fast and attention_writes_packed(q.dtype, ps, dh, single_rows, max_context, tiles_wide)),
           "attention: packed rows as out are written by the bfloat16 kernels only")
@@ -690,20 +695,22 @@ def attention(q, out, k_pool, v_pool, block_tables, tiles, n_heads, scale, windo
         part = torch.empty(n_tiles * n_heads * n_splits * (dh + 2) if n_splits > 1 else 1, dtype=torch.float32,
                            device=q.device)
         base = tiles.data_ptr()
-        _ok(lib.dn_attention_decode(
+        _ok(lib.dn_attention_decode_extras(
             q.data_ptr(), ldq, out.data_ptr(), ldo, k_pool.data_ptr(), v_pool.data_ptr(), block_tables.data_ptr(),
             block_tables.shape[1], base, base + 4 * n_tiles, base + 12 * n_tiles, n_tiles, part.data_ptr(), n_splits,
-            chunks, waves, n_heads, Hkv, dh, ps, float(scale), int(window), _stream()), "attention (decode)")
+            chunks, waves, n_heads, Hkv, dh, ps, float(scale), int(window), int(chunk), _ptr(bias), span, int(bool(sink)),
+            _stream()), "attention (decode)")
         return out
     if fast and tiles_wide is not None and dh in FLASH_HEAD_DIMS:
         _dev(tiles_wide, "tiles_wide", _I32, 2)
         _need(tiles_wide.is_contiguous() and tiles_wide.shape[0] == 4, "attention: tiles_wide")
         n_tiles = tiles_wide.shape[1]
         base = tiles_wide.data_ptr()
-        _ok(lib.dn_attention_flash(
+        _ok(lib.dn_attention_flash_extras(
             q.data_ptr(), ldq, out.data_ptr(), ldo, k_pool.data_ptr(), v_pool.data_ptr(), block_tables.data_ptr(),
             block_tables.shape[1], base, base + 4 * n_tiles, base + 8 * n_tiles, base + 12 * n_tiles, n_tiles,
-            n_heads, Hkv, dh, ps, float(scale), int(window), _stream()), "attention (flash)")
+            n_heads, Hkv, dh, ps, float(scale), int(window), int(chunk), _ptr(bias), span, int(bool(sink)), _stream()),
+            "attention (flash)")
         return out
     n_tiles = tiles.shape[1]
     base = tiles.data_ptr()
@@ -1268,7 +1275,7 @@ def gate_scan(a, b, g, bias_a, bias_b, state, row_start, slots, out):
     _f32vec(bias_a, "bias_a", width), _f32vec(bias_b, "bias_b", width)
     stride = _history(state, width, "gate_scan")
     _ok(_lib("sequence").dn_gate_scan(a.data_ptr(), _rows(a, "a"), b.data_ptr(), _rows(b, "b"), g.data_ptr(), _rows(g, "g"), _ptr(bias_a),
-                                      _ptr(bias_b), state.data_ptr(), stride, row_start.data_ptr(), slots.data_ptr(), S, width,
+                                      _ptr(bias_b), state.data_ptr(), stride, row_start.data_ptr(), slots.data_ptr(), S, T, width,
                                       out.data_ptr(), _CODE[out.dtype], _rows(out, "out"), _stream()), "gate_scan")
     return out
 
@@ -1302,21 +1309,51 @@ def streams_read(xs, w_in, weight, eps, out, rows=None):
     return out
 
 
-def streams_write(xs, y, mix, w_out, next_in=None, weight=None, eps=0.0, out=None):
+def streams_write(xs, y, mix, w_out, next_in=None, weight=None, eps=0.0, out=None, branches=None):
     """Every copy anew from the old ones and a sublayer's result: xs[t] <- sum_s mix[s, t] xs[s] + w_out[t] * y, in place.
-    next_in given: the same kernel then reads the new copies as streams_read(xs, next_in, weight, eps, out) does."""
+    next_in given: the same kernel then reads the new copies as streams_read(xs, next_in, weight, eps, out) does.
+    branches = (y2, w1, w2, eps): the result is the mean of two branches, each normed over the width first with a weight of its
+    own: (y / rms(y) * w1 + y2 / rms(y2) * w2) / 2, as two calls of rmsnorm_add with mult 1/2 into zeros make it."""
     n, T, width = _streams(xs, "streams_write")
     _dev(y, "y", (torch.float32,), 2)
     _need(tuple(y.shape) == (T, width), "streams_write: y")
     _f32vec(mix, "mix", n * n), _f32vec(w_out, "w_out", n), _f32vec(next_in, "next_in", n), _f32vec(weight, "weight", width)
+    y2 = w1 = w2 = None
+    beps = 0.0
+    if branches is not None:
+        y2, w1, w2, beps = branches
+        _dev(y2, "y2", (torch.float32,), 2)
+        _need(tuple(y2.shape) == (T, width), "streams_write: the second branch")
+        _f32vec(w1, "w1", width), _f32vec(w2, "w2", width)
     if next_in is not None:
         _dev(out, "out", _FLOATS, 2)
         _need(tuple(out.shape) == (T, width), "streams_write: out")
     _ok(_lib("sequence").dn_streams_write(xs.data_ptr(), T * width, n, mix.data_ptr(), w_out.data_ptr(), y.data_ptr(), _rows(y, "y"),
+                                          _ptr(y2), _rows(y2, "y2") if y2 is not None else 0, _ptr(w1), _ptr(w2), float(beps),
                                           _ptr(next_in), _ptr(weight), float(eps), _ptr(out) if next_in is not None else 0,
                                           _CODE[out.dtype] if next_in is not None else 0,
                                           _rows(out, "out") if next_in is not None else 0, T, width, _stream()), "streams_write")
     return out
+
+
+def norm_pair_write(z, q_width, wq, wk, eps, q_out, slot_map, k_pool, v_pool, write=True):
+    """A row of z (32-bit) is [q: q_width | k: the rest].  q_out = q / sqrt(mean(q^2) + eps) * wq; the key that goes to the cache
+    (k_pool [pages, Hkv, page, dh]) is k / sqrt(mean(k^2) + eps) * wk, each normed as one vector over all heads; the value
+    (v_pool [pages, Hkv, dh, page]) is k as it is.  slot_map: int32 [T], page * page_size + offset, negative: not written."""
+    _dev(z, "z", (torch.float32,), 2), _dev(q_out, "q_out", _FLOATS, 2), _dev(slot_map, "slot_map", _I32, 1)
+    _dev(k_pool, "k_pool", (q_out.dtype,), 4), _dev(v_pool, "v_pool", (q_out.dtype,), 4)
+    T = z.shape[0]
+    n_pages, Hkv, ps, dh = k_pool.shape
+    kw = z.shape[1] - q_width
+    _need(kw == Hkv * dh and q_width >= 1 and tuple(q_out.shape) == (T, q_width) and slot_map.is_contiguous() and slot_map.shape[0] == T,
+          "norm_pair_write: shapes")
+    _need(k_pool.is_contiguous() and v_pool.is_contiguous() and tuple(v_pool.shape) == (n_pages, Hkv, dh, ps), "norm_pair_write: pools")
+    _f32vec(wq, "wq", q_width), _f32vec(wk, "wk", kw)
+    _ok(_lib("sequence").dn_norm_pair_write(z.data_ptr(), _rows(z, "z"), q_width, kw, wq.data_ptr(), wk.data_ptr(), float(eps),
+                                            q_out.data_ptr(), _rows(q_out, "q_out"), slot_map.data_ptr(), k_pool.data_ptr(),
+                                            v_pool.data_ptr(), T, Hkv, dh, ps, _CODE[q_out.dtype], int(bool(write)), _stream()),
+        "norm_pair_write")
+    return q_out
 
 
 # -- a matrix per head, a matrix per expert (csrc/kernels/grouped.hip) -----------------------------------------------------

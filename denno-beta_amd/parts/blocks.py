@@ -216,15 +216,17 @@ class MultiStreamBlock:
         runtime.stream_rows = None
         h = came if came is not None else self.hc1.read(xs, self.norm1, act)
         cache = caches if len(caches) != 1 else caches[0]
-        y = SandwichBlock._result(self.mixer, xs[0], h, ctx, cache)
+        # (a mixer of two branches hands both results over: their norms and their mean happen in the write's kernel)
+        pair = self.mixer.forward_pair(h, ctx, caches) if hasattr(self.mixer, "forward_pair") else None
+        y, branches = pair if pair is not None else (SandwichBlock._result(self.mixer, xs[0], h, ctx, cache), None)
         nxt = getattr(runtime, "next_read", None)
         if self.has_ffn:
-            h = self.hc1.write(xs, y, self.hc2, self.norm2, act)
-            y = SandwichBlock._result(self.ffn, xs[0], h, ctx)
+            h = self.hc1.write(xs, y, self.hc2, self.norm2, act, branches=branches)
+            y, branches = SandwichBlock._result(self.ffn, xs[0], h, ctx), None
             last = self.hc2
         else:
             last = self.hc1
         if nxt is not None:
-            runtime.stream_rows = last.write(xs, y, nxt[0], nxt[1], act)
+            runtime.stream_rows = last.write(xs, y, nxt[0], nxt[1], act, branches=branches)
         else:
-            last.write(xs, y)
+            last.write(xs, y, branches=branches)

@@ -37,11 +37,13 @@ class StreamMixer(Part):
         out = torch.empty(xs.shape[1:], dtype=out_dtype, device=xs.device)
         return ops.streams_read(xs, self.w_in, norm.weight, norm.eps, out)
 
-    def write(self, xs, y, then=None, norm=None, out_dtype=None):
+    def write(self, xs, y, then=None, norm=None, out_dtype=None, branches=None):
         """The copies anew, in place.  then: the connector of the sublayer that reads the stream next; its read (with `norm`)
-        then happens in the same kernel and its rows come back."""
+        then happens in the same kernel and its rows come back.  branches: y is the first of two results whose normed mean
+        is the sublayer's (ops.streams_write)."""
         if then is None:
-            ops.streams_write(xs, y, self.mix, self.w_out)
+            ops.streams_write(xs, y, self.mix, self.w_out, branches=branches)
             return None
         out = torch.empty(xs.shape[1:], dtype=out_dtype, device=xs.device)
-        return ops.streams_write(xs, y, self.mix, self.w_out, next_in=then.w_in, weight=norm.weight, eps=norm.eps, out=out)
+        return ops.streams_write(xs, y, self.mix, self.w_out, next_in=then.w_in, weight=norm.weight, eps=norm.eps, out=out,
+                                 branches=branches)

@@ -345,13 +345,9 @@ class ChunkAttention(Part):
         H, G, d, qw, kw = self.n_heads, self.n_kv_heads, self.head_dim, self.q_width, self.kv_width
         g = ctx.groups[cache.group]
         z = self.proj(h, out_dtype=torch.float32)
-        q = torch.empty((T, qw), dtype=act, device=dev)
-        kv = torch.empty((T, 2 * kw), dtype=act, device=dev)      # normed keys at column 0, the projection as values at kw
-        ops.rmsnorm(z[:, :qw], self.q_norm, self.eps, q)
-        ops.rmsnorm(z[:, qw:], self.k_norm, self.eps, kv[:, :kw])
-        ops.rotary(z, kv, ctx.positions, self.no_freq, G, 0, d, src_off=qw, dst_off=kw)      # (moved, not turned)
-        if cache.writes:
-            ops.kv_write(kv, 0, kw, g.slot_map, cache.k, cache.v)
+        # one kernel: both norms, the normed keys and the projection as values to their places in the cache
+        q = ops.norm_pair_write(z, qw, self.q_norm, self.k_norm, self.eps, torch.empty((T, qw), dtype=act, device=dev), g.slot_map,
+                                cache.k, cache.v, write=cache.writes)
         o = torch.empty((T, qw), dtype=act, device=dev)
         ops.attention(q, o, cache.k, cache.v, g.block_tables, g.tiles, H, self.scale, 0, tiles_wide=g.tiles_wide,
                       single_rows=g.single_rows, max_context=g.max_context, chunk=self.chunk, bias=self.bias, sink=self.sink)
@@ -393,6 +389,14 @@ class ParallelMixers(Part):
         for b in self.branches:
             b.bind(tensors, runtime)
         self.norms = [tensors[n] for n in self.norm_names]
+
+    def forward_pair(self, h, ctx, caches):
+        """For two branches: -> (first result, (second result, first weight, second weight, eps)): whoever adds the
+        result into the stream norms and halves both in its own kernel (ops.streams_write's `branches`); None otherwise."""
+        if len(self.branches) != 2:
+            return None
+        a, b = (br.forward(h, ctx, cache, accumulate_into=None) for br, cache in zip(self.branches, caches))
+        return a, (b, self.norms[0], self.norms[1], self.eps)
 
     def forward(self, h, ctx, caches, accumulate_into):
         if not isinstance(caches, (list, tuple)):

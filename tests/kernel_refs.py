@@ -459,15 +459,32 @@ def streams_read(xs, w_in, weight, eps, out, rows=None):
     return out
 
 
-def streams_write(xs, y, mix, w_out, next_in=None, weight=None, eps=0.0, out=None):
+def streams_write(xs, y, mix, w_out, next_in=None, weight=None, eps=0.0, out=None, branches=None):
     n = xs.shape[0]
     old = xs.double().clone()
+    if branches is not None:
+        y2, w1, w2, beps = branches
+        unit = lambda v: v.double() / torch.sqrt((v.double() ** 2).mean(dim=-1, keepdim=True) + beps)      # noqa: E731
+        y = 0.5 * (unit(y) * w1.double() + unit(y2) * w2.double())
     m = mix.double().view(n, n)
     for t in range(n):
         xs[t] = (sum(m[s, t] * old[s] for s in range(n)) + w_out[t].double() * y.double()).to(xs.dtype)
     if next_in is not None:
         streams_read(xs, next_in, weight, eps, out)
     return out
+
+
+def norm_pair_write(z, q_width, wq, wk, eps, q_out, slot_map, k_pool, v_pool, write=True):
+    n_pages, hkv, ps, dh = k_pool.shape
+    unit = lambda v: v.double() / torch.sqrt((v.double() ** 2).mean(dim=-1, keepdim=True) + eps)      # noqa: E731
+    q_out.copy_(unit(z[:, :q_width]) * wq.double())
+    if write:
+        keys = (unit(z[:, q_width:]) * wk.double()).to(k_pool.dtype)
+        for t, slot in enumerate(slot_map.tolist()):
+            if slot >= 0:
+                k_pool[slot // ps, :, slot % ps, :] = keys[t].view(hkv, dh)
+                v_pool[slot // ps, :, :, slot % ps] = z[t, q_width:].view(hkv, dh).to(v_pool.dtype)
+    return q_out
 
 
 def pair_rows(tokens, positions, row_start, slots, last, mul_prev, mul_cur, buckets, out, write=True):

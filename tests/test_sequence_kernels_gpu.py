@@ -28,7 +28,8 @@ def tables(lengths, slots):
 def both(fn_name, make, outs, dtype=torch.float32):
     """Runs ops.<fn> on the device and kernel_refs.<fn> on copies on the host; compares the tensors named in `outs`."""
     args = make()
-    host = [a.detach().cpu().clone() if isinstance(a, torch.Tensor) else a for a in args]
+    cpu = lambda a: a.detach().cpu().clone() if isinstance(a, torch.Tensor) else a      # noqa: E731
+    host = [tuple(cpu(x) for x in a) if isinstance(a, tuple) else cpu(a) for a in args]
     getattr(ops, fn_name)(*args)
     getattr(ref, fn_name)(*host)
     torch.cuda.synchronize()
@@ -507,3 +508,42 @@ def test_rows_picked_by_pairs_of_tokens():
                              torch.empty(T, dtype=torch.int32), write)
         assert torch.equal(got.cpu()[:7], want[:7]) and torch.equal(got.cpu()[9:], want[9:]) and torch.equal(last_d.cpu(), last_h)
         assert got.cpu()[7:9].tolist() == [30011, 30011]      # (padding at position 0: the table's last row, no state touched)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("n,width", [(2, 96), (3, 1030)])
+def test_a_write_that_norms_two_branches(dtype, n, width):
+    T = 6
+    xs = torch.randn(n, T, width, device=DEV)
+    w_in, w_out, mix = torch.randn(n, device=DEV), torch.randn(n, device=DEV), torch.randn(n, n, device=DEV)
+    g, w1, w2 = torch.randn(width, device=DEV), torch.randn(width, device=DEV), torch.randn(width, device=DEV)
+    y1, y2 = torch.randn(T, width, device=DEV) * 3, torch.randn(T, width, device=DEV) * 0.2
+    both("streams_write", lambda: (xs.clone(), y1, mix, w_out, None, None, 0.0, None, (y2, w1, w2, 1e-5)), [0])
+    both("streams_write", lambda: (xs.clone(), y1, mix, w_out, w_in, g, 1e-6, torch.empty(T, width, dtype=dtype, device=DEV),
+                                   (y2, w1, w2, 1e-5)), [0, 7], dtype)
+    # the same bits as the norms as kernels of their own, added one after the other into zeros
+    a, b = xs.clone(), xs.clone()
+    ops.streams_write(a, y1, mix, w_out, branches=(y2, w1, w2, 1e-5))
+    y = torch.zeros(T, width, device=DEV)
+    ops.rmsnorm_add(y1, w1, None, 0.5, 1e-5, y), ops.rmsnorm_add(y2, w2, None, 0.5, 1e-5, y)
+    ops.streams_write(b, y, mix, w_out)
+    assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("H,Hkv,dh,ps", [(4, 2, 16, 16), (3, 1, 24, 8), (8, 8, 96, 16), (2, 2, 10, 4)])
+def test_queries_and_keys_normed_whole_and_written_to_the_cache(dtype, H, Hkv, dh, ps):
+    T, n_pages = 9, 5
+    z = torch.randn(T, (H + Hkv) * dh, device=DEV) * 2
+    wq, wk = torch.randn(H * dh, device=DEV), torch.randn(Hkv * dh, device=DEV)
+    places = torch.randperm(n_pages * ps)[:T].to(torch.int32)
+    places[3] = -1
+    slot_map = places.to(DEV)
+
+    def make():
+        return (z, H * dh, wq, wk, 1e-5, torch.empty(T, H * dh, dtype=dtype, device=DEV), slot_map,
+                torch.zeros(n_pages, Hkv, ps, dh, dtype=dtype, device=DEV), torch.zeros(n_pages, Hkv, dh, ps, dtype=dtype, device=DEV))
+    both("norm_pair_write", make, [5, 7, 8], dtype)
+    args = make() + (False,)
+    ops.norm_pair_write(*args)
+    assert float(args[7].float().abs().sum()) == 0.0 and float(args[8].float().abs().sum()) == 0.0
