@@ -421,7 +421,8 @@ def test_conv_with_a_bias(taps):
     both("conv_rows", lambda: (h, w, hist, row_start, slots, torch.zeros(T, width, device=DEV), False, "silu", b), [5])
 
 
-@pytest.mark.parametrize("dk,dv,heads,groups", [(16, 8, 4, 2), (48, 48, 6, 1), (24, 12, 3, 3), (128, 64, 2, 1), (6, 10, 2, 1)])
+@pytest.mark.parametrize("dk,dv,heads,groups", [(16, 8, 4, 2), (48, 48, 6, 1), (24, 12, 3, 3), (128, 64, 2, 1), (6, 10, 2, 1),
+                                                (128, 32, 64, 2), (64, 16, 128, 1), (100, 20, 64, 4)])
 @pytest.mark.parametrize("lengths", [[1, 1, 1], [5, 40, 1, 17]])
 def test_state_scan_with_a_decay_per_row_and_head(dk, dv, heads, groups, lengths):
     row_start, slots, T = tables(lengths, list(range(len(lengths)))[::-1])
