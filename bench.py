@@ -323,7 +323,7 @@ def dogalorn_configs(width, layers=4, vocab=32000, positions=2048):
     mam = dict(type="mamba2", mlp=ff, mixer=dict(heads=2 * H, vdim=64, state=128, groups=1, conv=4, norm_groups=1))
     kinds = [par, mam, mam, par]
     dog = dict(architecture="Dogalorn", vocab=vocab, width=width, norm=dict(eps=1e-5), streams=2, logit_scale=1.0,
-               embedding=dict(bigram=dict(buckets=100003, mul_prev=31, mul_cur=17)), layers=[kinds[i % 4] for i in range(layers)],
+               embedding=dict(bigram=dict(buckets=100003, mul_prev=7919, mul_cur=4099)), layers=[kinds[i % 4] for i in range(layers)],
                max_positions=positions, n_positions=positions, vocab_size=vocab)
     Hl = width // 128
     att = dict(type="attention", mlp=ff, mixer=dict(heads=H, kv_heads=max(1, H // 4), dim=64, vdim=64, scale=0.125,
