@@ -815,6 +815,83 @@ __global__ __launch_bounds__(256) void streams_write_kernel(float* xs, size_t pl
   }
 }
 
+// streams_write_kernel for rows of up to 256 NC columns and up to NS copies: a thread's share of the row (the copies, the
+// result, the branches' weights) is asked for at once and stays in registers from the first sum to the last store, where the
+// kernel above goes to memory three times one behind the other: a decode step's rows wait for those trips, not for bytes.
+// The same sums in the same order: the same bits.
+template <int NS, int NC>
+__global__ __launch_bounds__(256) void streams_write_held_kernel(float* xs, size_t plane, int n, const float* mix, const float* w_out,
+                                                                 const float* y, size_t ldy, const float* y2, size_t ldy2, const float* by,
+                                                                 const float* by2, float beps, const float* next_in, const float* g,
+                                                                 float eps, void* out, int out_dt, size_t ldo, int width) {
+  __shared__ float sh[4];
+  __shared__ float sm[STREAMS_MAX * STREAMS_MAX + 2 * STREAMS_MAX];
+  const size_t row = blockIdx.x;
+  float old[NS][NC], yv[NC], y2v[NC], b1[NC], b2[NC], gv[NC];
+#pragma unroll
+  for (int k = 0; k < NC; ++k) {
+    const int c = threadIdx.x + 256 * k;
+    const bool ok = c < width;
+    const int cc = ok ? c : 0;
+    yv[k] = ok ? y[row * ldy + cc] : 0.f;
+    y2v[k] = (y2 && ok) ? y2[row * ldy2 + cc] : 0.f;
+    b1[k] = y2 ? by[cc] : 0.f, b2[k] = y2 ? by2[cc] : 0.f;
+    gv[k] = (next_in && g) ? g[cc] : 1.0f;
+#pragma unroll
+    for (int s = 0; s < NS; ++s) old[s][k] = (s < n && ok) ? xs[s * plane + row * width + cc] : 0.f;
+  }
+  if (threadIdx.x < n * n) sm[threadIdx.x] = mix[threadIdx.x];
+  if (threadIdx.x < n) {
+    sm[STREAMS_MAX * STREAMS_MAX + threadIdx.x] = w_out[threadIdx.x];
+    sm[STREAMS_MAX * STREAMS_MAX + STREAMS_MAX + threadIdx.x] = next_in ? next_in[threadIdx.x] : 0.f;
+  }
+  __syncthreads();
+  const float* wo = sm + STREAMS_MAX * STREAMS_MAX;
+  const float* wn = wo + STREAMS_MAX;
+  if (y2) {
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int k = 0; k < NC; ++k) s1 = fmaf(yv[k], yv[k], s1), s2 = fmaf(y2v[k], y2v[k], s2);
+    s1 = block_sum_256(s1, sh);
+    s2 = block_sum_256(s2, sh);
+    const float inv1 = 1.0f / sqrtf(s1 / static_cast<float>(width) + beps), inv2 = 1.0f / sqrtf(s2 / static_cast<float>(width) + beps);
+#pragma unroll
+    for (int k = 0; k < NC; ++k) yv[k] = fmaf(0.5f, y2v[k] * inv2 * b2[k], fmaf(0.5f, yv[k] * inv1 * b1[k], 0.f));
+  }
+  float ss = 0.f, u[NC];
+#pragma unroll
+  for (int k = 0; k < NC; ++k) {
+    const int c = threadIdx.x + 256 * k;
+    u[k] = 0.f;
+    if (c < width) {
+#pragma unroll
+      for (int t = 0; t < NS; ++t) {
+        if (t < n) {
+          float acc = 0.f;
+#pragma unroll
+          for (int s = 0; s < NS; ++s)
+            if (s < n) acc = fmaf(sm[s * n + t], old[s][k], acc);
+          acc = fmaf(wo[t], yv[k], acc);
+          xs[t * plane + row * width + c] = acc;
+          u[k] = fmaf(wn[t], acc, u[k]);
+        }
+      }
+      ss = fmaf(u[k], u[k], ss);
+    }
+  }
+  if (!next_in) return;
+  ss = block_sum_256(ss, sh);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(width) + eps);
+#pragma unroll
+  for (int k = 0; k < NC; ++k) {
+    const int c = threadIdx.x + 256 * k;
+    if (c < width) {
+      const float v = u[k] * inv;
+      store_as(out, row * ldo + c, out_dt, g ? v * gv[k] : v);
+    }
+  }
+}
+
 bool float_kind(int dt) { return dt == DN_F32 || dt == DN_BF16; }
 
 }  // namespace
@@ -1072,9 +1149,21 @@ int dn_streams_write(float* xs, long long plane, int n, const float* mix, const 
   if (next_in && !float_kind(out_dt)) return DN_ERR_DTYPE;
   if (n < 1 || n > STREAMS_MAX || width < 1 || (next_in && !out) || (y2 && (!by || !by2))) return DN_ERR_SHAPE;
   if (T == 0) return 0;
-  hipLaunchKernelGGL(streams_write_kernel, dim3(T), dim3(256), 0, stream, xs, static_cast<size_t>(plane), n, mix, w_out, y,
-                     static_cast<size_t>(ldy), y2, static_cast<size_t>(ldy2), by, by2, beps, next_in, g, eps, out, out_dt,
-                     static_cast<size_t>(ldo), width);
+#define DN_STREAMS_HELD(NS, NC)                                                                                              \
+  hipLaunchKernelGGL((streams_write_held_kernel<NS, NC>), dim3(T), dim3(256), 0, stream, xs, static_cast<size_t>(plane), n, mix,    \
+                     w_out, y, static_cast<size_t>(ldy), y2, static_cast<size_t>(ldy2), by, by2, beps, next_in, g, eps, out, out_dt, \
+                     static_cast<size_t>(ldo), width)
+  // (up to 4 copies of rows up to 4,096 wide: a thread holds its share of the row; by the sizes alone, the same bits either way)
+  if (n <= 2 && width <= 1024) DN_STREAMS_HELD(2, 4);
+  else if (n <= 2 && width <= 2048) DN_STREAMS_HELD(2, 8);
+  else if (n <= 4 && width <= 1024) DN_STREAMS_HELD(4, 4);
+  else if (n <= 4 && width <= 2048) DN_STREAMS_HELD(4, 8);
+  else if (n <= 4 && width <= 4096) DN_STREAMS_HELD(4, 16);
+  else
+    hipLaunchKernelGGL(streams_write_kernel, dim3(T), dim3(256), 0, stream, xs, static_cast<size_t>(plane), n, mix, w_out, y,
+                       static_cast<size_t>(ldy), y2, static_cast<size_t>(ldy2), by, by2, beps, next_in, g, eps, out, out_dt,
+                       static_cast<size_t>(ldo), width);
+#undef DN_STREAMS_HELD
   return dn_launch_status();
 }
 

@@ -476,7 +476,7 @@ def test_gate_scan(dtype, lengths, width):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("n,width", [(1, 40), (3, 256), (4, 77), (8, 1030)])
+@pytest.mark.parametrize("n,width", [(1, 40), (3, 256), (4, 77), (8, 1030), (2, 2000), (4, 3000), (2, 5000), (5, 300)])
 def test_a_stream_in_copies_read_and_written(dtype, n, width):
     T = 7
     xs = torch.randn(n, T, width, device=DEV)
