@@ -598,6 +598,41 @@ __global__ __launch_bounds__(256) void head_norm_wide_kernel(HeadNormArgs a) {
   }
 }
 
+// head_norm_wide_kernel for heads of up to 256 NC columns: a thread's share of the head stays in registers between the sum and
+// the stores (one trip to memory where the kernel above makes two).  The same sums in the same order: the same bits.
+template <int NC>
+__global__ __launch_bounds__(256) void head_norm_held_kernel(HeadNormArgs a) {
+  __shared__ float sh[4];
+  const int h = blockIdx.y, dv = a.dv;
+  const size_t t = blockIdx.x;
+  float y[NC], w[NC], gt[NC];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < NC; ++k) {
+    const int j = threadIdx.x + 256 * k;
+    const bool ok = j < dv;
+    const int jj = ok ? j : 0;
+    y[k] = ok ? head_norm_in(a, t, h * dv + jj) : 0.f;
+    w[k] = a.weight ? a.weight[h * a.w_stride + jj] : 1.0f;
+    gt[k] = (a.gate && !a.gate_first) ? a.gate[t * a.ldg + static_cast<size_t>(h) * dv + jj] : 0.f;
+  }
+#pragma unroll
+  for (int k = 0; k < NC; ++k)
+    if (threadIdx.x + 256 * k < dv) ss = fmaf(y[k], y[k], ss);
+  ss = block_sum_256(ss, sh);
+  const float inv = 1.0f / sqrtf(ss / static_cast<float>(dv) + a.eps);
+#pragma unroll
+  for (int k = 0; k < NC; ++k) {
+    const int j = threadIdx.x + 256 * k;
+    if (j < dv) {
+      float v = y[k] * inv;
+      if (a.weight) v *= w[k];
+      if (a.gate && !a.gate_first) v *= activation(a.gate_kind, gt[k], 0.f);
+      store_as(a.out, t * a.ldo + static_cast<size_t>(h) * dv + j, a.out_dt, v);
+    }
+  }
+}
+
 // ---- what a state-space recurrence with one decay per head reads -------------------------------------------------
 // dt = log(1 + e^(z[t, h] + bias[h])); decay[t, h] = exp(-rate[h] * dt); v[t, h, :] = dt * x[t, h, :].  A workgroup a row.
 __global__ __launch_bounds__(256) void step_sizes_kernel(const float* z, size_t ldz, const float* bias, const float* rate, const float* x,
@@ -1099,7 +1134,11 @@ int dn_head_norm(const float* o, long long ld, const float* weight, int w_stride
   if (T == 0) return 0;
   HeadNormArgs a{o, static_cast<size_t>(ld), weight, w_stride, eps, gate, static_cast<size_t>(ldg), gate_kind, gate_first, skip,
                  static_cast<size_t>(lds), skip_scale, skip_dim, out, out_dt, static_cast<size_t>(ldo), dv};
-  if (dv > 256)
+  if (dv > 256 && dv <= 2048)
+    hipLaunchKernelGGL(head_norm_held_kernel<8>, dim3(T, H), dim3(256), 0, stream, a);
+  else if (dv > 2048 && dv <= 4096)
+    hipLaunchKernelGGL(head_norm_held_kernel<16>, dim3(T, H), dim3(256), 0, stream, a);
+  else if (dv > 256)
     hipLaunchKernelGGL(head_norm_wide_kernel, dim3(T, H), dim3(256), 0, stream, a);
   else
     hipLaunchKernelGGL(head_norm_kernel, dim3(T, H), dim3(64), 0, stream, a);

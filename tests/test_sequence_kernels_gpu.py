@@ -439,7 +439,7 @@ def test_state_scan_with_a_decay_per_row_and_head(dk, dv, heads, groups, lengths
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("heads,dv", [(2, 24), (1, 300), (4, 16)])
+@pytest.mark.parametrize("heads,dv", [(2, 24), (1, 300), (4, 16), (1, 3000), (1, 5000), (2, 2048)])
 def test_head_norm_with_the_gate_first_and_a_second_summand(dtype, heads, dv):
     T, n = 9, heads * dv
     o, gate, skip = torch.randn(T, n, device=DEV), torch.randn(T, n, device=DEV), torch.randn(T, n, device=DEV)
