@@ -127,11 +127,16 @@ __global__ __launch_bounds__(64) void route_kernel(const float* z, size_t ldz, c
 
 // The same choice with a wave a row (up to 8,192 experts, `top` up to 64): lane l has the experts l, l + 64, ...; the
 // largest score is found over the lanes, the lowest index among equals wins, and lane c keeps the c-th choice.
+// groups > 1: the experts are `groups` equal runs of neighbours; a group's score is the sum of its two largest
+// s + correction (of its one, if it has one expert), and only the experts of the `keep` best groups (the lower index wins a
+// tie) can be chosen.  scale multiplies the weights.
 __global__ __launch_bounds__(64) void route_wave_kernel(const float* z, size_t ldz, const float* correction, int E, int top, int sigmoid,
-                                                        int renorm, int* ids, float* wts) {
+                                                        int renorm, int* ids, float* wts, int groups, int keep, float scale) {
   const int t = blockIdx.x, lane = threadIdx.x;
   const float* row = z + static_cast<size_t>(t) * ldz;
   const float none = -__builtin_huge_valf();
+  __shared__ unsigned char open_group[8192];      // (groups <= experts <= 8,192)
+  __shared__ float group_score[8192];
   float m = none;
   for (int e = lane; e < E; e += 64) m = fmaxf(m, row[e]);
   m = wave_max(m);
@@ -139,6 +144,36 @@ __global__ __launch_bounds__(64) void route_wave_kernel(const float* z, size_t l
   for (int e = lane; e < E; e += 64) sum += expf(row[e] - m);
   sum = wave_sum(sum);
   unsigned taken[4] = {0u, 0u, 0u, 0u};      // a bit for each of the lane's up to 128 experts
+  const int per = groups > 1 ? E / groups : E;
+  if (groups > 1) {
+    // lane l scores the groups l, l + 64, ...; then the best group is found `keep` times over the lanes
+    for (int g = lane; g < groups; g += 64) {
+      float first = none, second = none;
+      for (int e = g * per; e < (g + 1) * per; ++e) {
+        const float v = route_score(sigmoid, row[e], m, sum) + (correction ? correction[e] : 0.f);
+        if (v > first) second = first, first = v;
+        else if (v > second) second = v;
+      }
+      group_score[g] = per > 1 ? first + second : first;
+      open_group[g] = 0;
+    }
+    __syncthreads();
+    for (int c = 0; c < keep; ++c) {
+      float best_v = none;
+      int best = 0x7fffffff;
+      for (int g = lane; g < groups; g += 64)
+        if (!open_group[g] && group_score[g] > best_v) best_v = group_score[g], best = g;
+      const float top_v = wave_max(best_v);
+      int win = static_cast<int>(-wave_max(-static_cast<float>((best_v == top_v && best < groups) ? best : 16777216)));
+      if (win >= groups) {      // (scores that are no numbers: the first group that is still closed)
+        win = 0;
+        while (win < groups - 1 && open_group[win]) ++win;
+      }
+      __syncthreads();
+      if (lane == 0) open_group[win] = 1;
+      __syncthreads();
+    }
+  }
   float my_w = 0.f;
   int my_id = 0;
   for (int c = 0; c < top; ++c) {
@@ -146,6 +181,7 @@ __global__ __launch_bounds__(64) void route_wave_kernel(const float* z, size_t l
     int best = 0x7fffffff;
     for (int e = lane, k = 0; e < E; e += 64, ++k) {
       if ((taken[k >> 5] >> (k & 31)) & 1u) continue;
+      if (groups > 1 && !open_group[e / per]) continue;
       const float sc = route_score(sigmoid, row[e], m, sum);
       const float v = sc + (correction ? correction[e] : 0.f);
       if (v > best_v) best_v = v, best = e, best_s = sc;
@@ -161,7 +197,7 @@ __global__ __launch_bounds__(64) void route_wave_kernel(const float* z, size_t l
   const float chosen = wave_sum(lane < top ? my_w : 0.f);
   if (lane < top) {
     ids[t * top + lane] = my_id;
-    wts[t * top + lane] = renorm ? my_w / (chosen + 1e-20f) : my_w;
+    wts[t * top + lane] = (renorm ? my_w / (chosen + 1e-20f) : my_w) * scale;
   }
 }
 
@@ -262,6 +298,7 @@ __device__ __forceinline__ bool expert_tile(const int* offsets, int E, int id, i
 // kind 0: g * sigmoid(alpha g) * (u + 1) with g = min(W_gate h, limit), u = clamp(W_up h, +-limit)
 // kind 1: silu(s g) * (s u), s the pair's own factor (in_scale[pair]; none: 1): the expert reads s h, and both products
 //         are linear in what they read
+// kind 2: relu(s u)^2: an expert without a gate; the kernels are then built without the second product (DUAL false)
 struct ExpertAct {
   float limit, alpha;
   int kind;
@@ -273,10 +310,15 @@ __device__ __forceinline__ float expert_act(const ExpertAct& a, float g, float u
     const float gs = g * s;
     return gs / (1.0f + expf(-gs)) * (u * s);
   }
+  if (a.kind == 2) {      // (no gate: g is not computed)
+    const float r = fmaxf(u * s, 0.f);
+    return r * r;
+  }
   const float gv = fminf(g, a.limit), uv = fminf(fmaxf(u, -a.limit), a.limit);
   return gv / (1.0f + expf(-a.alpha * gv)) * (uv + 1.0f);
 }
 
+template <bool DUAL>
 __global__ __launch_bounds__(256) void expert_up_kernel(const void* h, int h_dt, size_t ldh, const int* order, const int* offsets,
                                                         int E, int top, const void* wg, const void* wu, int w_dt, int ff, int width,
                                                         ExpertAct act, void* y, int y_dt) {
@@ -291,7 +333,8 @@ __global__ __launch_bounds__(256) void expert_up_kernel(const void* h, int h_dt,
     a_row[q] = p < p1 ? static_cast<long long>(order[p] / top) * ldh : -1;
   }
   float g[4] = {0.f, 0.f, 0.f, 0.f}, u[4] = {0.f, 0.f, 0.f, 0.f};
-  tile_product<true>(lds, &lds2, h, h_dt, a_row, wg, wu, w_dt, static_cast<size_t>(e) * ff * width, ff, width, n0, g, u);
+  if (DUAL) tile_product<true>(lds, &lds2, h, h_dt, a_row, wg, wu, w_dt, static_cast<size_t>(e) * ff * width, ff, width, n0, g, u);
+  else tile_product<false>(lds, nullptr, h, h_dt, a_row, wu, nullptr, w_dt, static_cast<size_t>(e) * ff * width, ff, width, n0, u, nullptr);
   const int p = p0 + (tid >> 4);
   if (p >= p1) return;
   const float sc = act.in_scale ? act.in_scale[order[p]] : 1.0f;
@@ -451,6 +494,7 @@ __device__ __forceinline__ bool expert_tile64(const int* offsets, int E, int id,
   return false;
 }
 
+template <bool DUAL>
 __global__ __launch_bounds__(256) void expert_up_mfma_kernel(const bf16_t* h, size_t ldh, const int* order, const int* offsets, int E,
                                                              int top, const bf16_t* wg, const bf16_t* wu, int ff, int width,
                                                              ExpertAct act, bf16_t* y, int tiles_x) {
@@ -467,11 +511,12 @@ __global__ __launch_bounds__(256) void expert_up_mfma_kernel(const bf16_t* h, si
     const int p = min(pw + 16 * i + lr, p1 - 1);
     a_ptr[i] = h + static_cast<size_t>(order[p] / top) * ldh + kq;
     const size_t n = min(nw + 16 * i + lr, ff - 1);
-    g_ptr[i] = wg + (static_cast<size_t>(e) * ff + n) * width + kq;
+    g_ptr[i] = DUAL ? wg + (static_cast<size_t>(e) * ff + n) * width + kq : nullptr;
     u_ptr[i] = wu + (static_cast<size_t>(e) * ff + n) * width + kq;
   }
   f32x4 g[2][2] = {}, u[2][2] = {};
-  mfma_tile<true, false, 2>(a_ptr, g_ptr, u_ptr, width, g, u);
+  if (DUAL) mfma_tile<true, false, 2>(a_ptr, g_ptr, u_ptr, width, g, u);
+  else mfma_tile<false, false, 2>(a_ptr, u_ptr, nullptr, width, u, nullptr);
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int p = pw + 16 * i + lr;
@@ -526,7 +571,7 @@ __global__ __launch_bounds__(256) void expert_down_mfma_kernel(const bf16_t* y, 
 // multiple of 16): a wave takes 32 pairs x 64 columns, a workgroup 64 x 128; where the step has few pairs an expert
 // (decoded tokens: the kernel then only streams the chosen experts' matrices) a wave takes 16 columns, so that four
 // times as many waves have loads in flight.  An element's sum is the same in both.
-template <int CB>
+template <int CB, bool DUAL>
 __global__ __launch_bounds__(256) void expert_up_packed_kernel(const bf16_t* h, size_t ldh, const int* order, const int* offsets, int E,
                                                                int top, const bf16_t* wg, const bf16_t* wu, int ff, int width,
                                                                ExpertAct act, bf16_t* y, int tiles_x) {
@@ -545,11 +590,12 @@ __global__ __launch_bounds__(256) void expert_up_packed_kernel(const bf16_t* h, 
 #pragma unroll
   for (int j = 0; j < CB; ++j) {
     const size_t block = (static_cast<size_t>(e) * ff + min(nw + 16 * j, ff - 16)) / 16;
-    g_ptr[j] = wg + block * ksteps * 512 + lane * 8;
+    g_ptr[j] = DUAL ? wg + block * ksteps * 512 + lane * 8 : nullptr;
     u_ptr[j] = wu + block * ksteps * 512 + lane * 8;
   }
   f32x4 g[2][CB] = {}, u[2][CB] = {};
-  mfma_tile_staged<true, CB>(stage[wave], a_ptr, g_ptr, u_ptr, width, g, u);
+  if (DUAL) mfma_tile_staged<true, CB>(stage[wave], a_ptr, g_ptr, u_ptr, width, g, u);
+  else mfma_tile_staged<false, CB>(stage[wave], a_ptr, u_ptr, nullptr, width, u, nullptr);
 #pragma unroll
   for (int i = 0; i < 2; ++i) {
     const int p = pw + 16 * i + lr;
@@ -685,14 +731,16 @@ int dn_heads_linear(const void* a, int a_dt, long long lda, int a_off, int a_str
 }
 
 int dn_moe_route(const float* z, long long ldz, const float* correction, int T, int E, int top, int sigmoid, int renorm, int* ids,
-                 float* wts, hipStream_t stream) {
+                 float* wts, int groups, int keep, float scale, hipStream_t stream) {
   if (E < 1 || top < 1 || top > E || ldz < E) return DN_ERR_SHAPE;
+  if (groups < 1 || E % groups != 0 || keep < 1 || keep > groups || top > keep * (E / groups)) return DN_ERR_SHAPE;
   if (T == 0) return 0;
   if (E <= 8192 && top <= 64) {
     hipLaunchKernelGGL(route_wave_kernel, dim3(T), dim3(64), 0, stream, z, static_cast<size_t>(ldz), correction, E, top, sigmoid, renorm,
-                       ids, wts);
+                       ids, wts, keep < groups ? groups : 1, keep, scale);
     return dn_launch_status();
   }
+  if (keep < groups || scale != 1.0f) return DN_ERR_SHAPE;      // (the kernel of a thread a row knows neither)
   hipLaunchKernelGGL(route_kernel, dim3((T + 63) / 64), dim3(64), 0, stream, z, static_cast<size_t>(ldz), correction, T, E, top, sigmoid,
                      renorm, ids, wts);
   return dn_launch_status();
@@ -711,35 +759,47 @@ int dn_moe_up(const void* h, int h_dt, long long ldh, const int* order, const in
               const void* wu, int w_dt, int ff, int width, float limit, float alpha, int kind, const float* in_scale, void* y,
               int y_dt, int packed, hipStream_t stream) {
   if (!float_kind(h_dt) || !float_kind(w_dt) || !float_kind(y_dt)) return DN_ERR_DTYPE;
-  if (kind < 0 || kind > 1) return DN_ERR_SHAPE;
+  if (kind < 0 || kind > 2) return DN_ERR_SHAPE;
+  const bool dual = kind != 2;
   if (n == 0) return 0;
   const ExpertAct act{limit, alpha, kind, in_scale};
   if (packed) {
     if (h_dt != DN_BF16 || w_dt != DN_BF16 || y_dt != DN_BF16) return DN_ERR_DTYPE;
-    if (width % 32 != 0 || ff % 16 != 0 || ldh % 8 != 0 || !aligned16(h) || !aligned16(wg) || !aligned16(wu)) return DN_ERR_SHAPE;
+    if (width % 32 != 0 || ff % 16 != 0 || ldh % 8 != 0 || !aligned16(h) || (dual && !aligned16(wg)) || !aligned16(wu)) return DN_ERR_SHAPE;
     const int tiles_x = (n + MT - 1) / MT + E;
     if (n <= 16 * E) {
       const int tiles = tiles_x * ((ff + 31) / 32);
-      hipLaunchKernelGGL(expert_up_packed_kernel<1>, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(h),
+      if (dual) hipLaunchKernelGGL((expert_up_packed_kernel<1, true>), dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(h),
+                         static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg),
+                         static_cast<const bf16_t*>(wu), ff, width, act, static_cast<bf16_t*>(y), tiles_x);
+      else hipLaunchKernelGGL((expert_up_packed_kernel<1, false>), dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(h),
                          static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg),
                          static_cast<const bf16_t*>(wu), ff, width, act, static_cast<bf16_t*>(y), tiles_x);
     } else {
       const int tiles = tiles_x * ((ff + 127) / 128);
-      hipLaunchKernelGGL(expert_up_packed_kernel<4>, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(h),
+      if (dual) hipLaunchKernelGGL((expert_up_packed_kernel<4, true>), dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(h),
+                         static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg),
+                         static_cast<const bf16_t*>(wu), ff, width, act, static_cast<bf16_t*>(y), tiles_x);
+      else hipLaunchKernelGGL((expert_up_packed_kernel<4, false>), dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream, static_cast<const bf16_t*>(h),
                          static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg),
                          static_cast<const bf16_t*>(wu), ff, width, act, static_cast<bf16_t*>(y), tiles_x);
     }
     return dn_launch_status();
   }
-  if (h_dt == DN_BF16 && w_dt == DN_BF16 && y_dt == DN_BF16 && width % 32 == 0 && ldh % 8 == 0 && aligned16(h) && aligned16(wg) &&
+  if (h_dt == DN_BF16 && w_dt == DN_BF16 && y_dt == DN_BF16 && width % 32 == 0 && ldh % 8 == 0 && aligned16(h) && (!dual || aligned16(wg)) &&
       aligned16(wu)) {
     const int tiles_x = (n + MT - 1) / MT + E, tiles = tiles_x * ((ff + 63) / 64);
-    hipLaunchKernelGGL(expert_up_mfma_kernel, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream,
+    if (dual) hipLaunchKernelGGL(expert_up_mfma_kernel<true>, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream,
+                       static_cast<const bf16_t*>(h), static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg),
+                       static_cast<const bf16_t*>(wu), ff, width, act, static_cast<bf16_t*>(y), tiles_x);
+  else hipLaunchKernelGGL(expert_up_mfma_kernel<false>, dim3((tiles + 7) / 8 * 8), dim3(256), 0, stream,
                        static_cast<const bf16_t*>(h), static_cast<size_t>(ldh), order, offsets, E, top, static_cast<const bf16_t*>(wg),
                        static_cast<const bf16_t*>(wu), ff, width, act, static_cast<bf16_t*>(y), tiles_x);
     return dn_launch_status();
   }
-  hipLaunchKernelGGL(expert_up_kernel, dim3((n + TM - 1) / TM + E, (ff + TN - 1) / TN), dim3(256), 0, stream, h, h_dt,
+  if (dual) hipLaunchKernelGGL(expert_up_kernel<true>, dim3((n + TM - 1) / TM + E, (ff + TN - 1) / TN), dim3(256), 0, stream, h, h_dt,
+                     static_cast<size_t>(ldh), order, offsets, E, top, wg, wu, w_dt, ff, width, act, y, y_dt);
+  else hipLaunchKernelGGL(expert_up_kernel<false>, dim3((n + TM - 1) / TM + E, (ff + TN - 1) / TN), dim3(256), 0, stream, h, h_dt,
                      static_cast<size_t>(ldh), order, offsets, E, top, wg, wu, w_dt, ff, width, act, y, y_dt);
   return dn_launch_status();
 }

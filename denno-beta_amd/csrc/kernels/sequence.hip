@@ -61,20 +61,26 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const void* x, int x_dt, s
 }
 
 // x[t, :] += mult * (y[t, :] / sqrt(mean(y^2) + eps) * weight) * scale: the norm of a sublayer's result, added into the
-// stream (scale: a vector, or none).  One workgroup a row, the sums as in rmsnorm_kernel.
+// stream (scale: a vector, or none).  gate: y is y * sigmoid(gate[t, :]) first, under the norm's sums too (a gate on the
+// sublayer's result).  One workgroup a row, the sums as in rmsnorm_kernel.
 __global__ __launch_bounds__(256) void rmsnorm_add_kernel(const void* y, int y_dt, size_t ldy, const float* weight, const float* scale,
-                                                          float mult, float* x, size_t ldx, int width, float eps) {
+                                                          float mult, float* x, size_t ldx, int width, float eps, const float* gate,
+                                                          size_t ldg) {
   __shared__ float sh[4];
   const size_t src = static_cast<size_t>(blockIdx.x) * ldy, dst = static_cast<size_t>(blockIdx.x) * ldx;
+  const float* g = gate ? gate + static_cast<size_t>(blockIdx.x) * ldg : nullptr;
   float ss = 0.f;
   for (int c = threadIdx.x; c < width; c += 256) {
-    const float v = load_as(y, src + c, y_dt);
+    float v = load_as(y, src + c, y_dt);
+    if (g) v *= 1.0f / (1.0f + expf(-g[c]));
     ss = fmaf(v, v, ss);
   }
   ss = block_sum_256(ss, sh);
   const float inv = 1.0f / sqrtf(ss / static_cast<float>(width) + eps);
   for (int c = threadIdx.x; c < width; c += 256) {
-    float v = load_as(y, src + c, y_dt) * inv;
+    float v = load_as(y, src + c, y_dt);
+    if (g) v *= 1.0f / (1.0f + expf(-g[c]));
+    v *= inv;
     if (weight) v *= weight[c];
     if (scale) v *= scale[c];
     x[dst + c] = fmaf(mult, v, x[dst + c]);
@@ -226,10 +232,12 @@ __global__ __launch_bounds__(256) void shift_mix_kernel(const void* h, int h_dt,
 
 // ---- pairs of dimensions turned by the position ------------------------------------------------------------
 // Vector n of row t starts at src_off + n * src_stride; its entries 2i and 2i + 1 (i < dims / 2) are turned by the
-// angle position * freq[i], the other `width - dims` entries pass; the result goes to dst_off + n * dst_stride.
+// angle position * freq[i] (cos and sin times `mag`: a scaled encoding's factor, 1 otherwise), the other `width - dims`
+// entries pass; the result goes to dst_off + n * dst_stride.
 __global__ __launch_bounds__(256) void rotary_kernel(const void* src, int src_dt, size_t ld_src, int src_off, int src_stride,
                                                      void* dst, int dst_dt, size_t ld_dst, int dst_off, int dst_stride,
-                                                     const int* positions, const float* freq, int n_vec, int dims, int width) {
+                                                     const int* positions, const float* freq, int n_vec, int dims, int width,
+                                                     float mag) {
   const int t = blockIdx.x;
   const float p = static_cast<float>(positions[t]);
   const int half = dims / 2, rest = width - dims;
@@ -240,7 +248,7 @@ __global__ __launch_bounds__(256) void rotary_kernel(const void* src, int src_dt
     const size_t b = static_cast<size_t>(t) * ld_dst + dst_off + static_cast<size_t>(n) * dst_stride;
     if (i < half) {
       const float ang = p * freq[i];
-      const float c = cosf(ang), sn = sinf(ang);
+      const float c = cosf(ang) * mag, sn = sinf(ang) * mag;
       const float u = load_as(src, a + 2 * i, src_dt), v = load_as(src, a + 2 * i + 1, src_dt);
       store_as(dst, b + 2 * i, dst_dt, u * c - v * sn);
       store_as(dst, b + 2 * i + 1, dst_dt, v * c + u * sn);
@@ -258,6 +266,7 @@ struct TurnRun {
   int dst_dt;
   size_t ld_dst;
   int src_off, dst_off, dst_stride, n_vec, width, dims;      // (src_stride is the width: the vectors lie side by side)
+  int unit;      // the vectors are divided by their root mean square behind the turn (rotary_runs_unit_kernel)
 };
 struct TurnRuns {
   TurnRun run[3];
@@ -265,7 +274,7 @@ struct TurnRuns {
 };
 
 __global__ __launch_bounds__(256) void rotary_runs_kernel(const void* src, int src_dt, size_t ld_src, TurnRuns runs, const int* positions,
-                                                          const float* freq) {
+                                                          const float* freq, float mag) {
   const int t = blockIdx.x;
   const float p = static_cast<float>(positions[t]);
   for (int r = 0; r < runs.n; ++r) {
@@ -277,7 +286,7 @@ __global__ __launch_bounds__(256) void rotary_runs_kernel(const void* src, int s
       const size_t b = static_cast<size_t>(t) * u.ld_dst + u.dst_off + static_cast<size_t>(n) * u.dst_stride;
       if (i < half) {
         const float ang = p * freq[i];
-        const float c = cosf(ang), sn = sinf(ang);
+        const float c = cosf(ang) * mag, sn = sinf(ang) * mag;
         const float x = load_as(src, a + 2 * i, src_dt), y = load_as(src, a + 2 * i + 1, src_dt);
         store_as(u.dst, b + 2 * i, u.dst_dt, x * c - y * sn);
         store_as(u.dst, b + 2 * i + 1, u.dst_dt, y * c + x * sn);
@@ -289,8 +298,74 @@ __global__ __launch_bounds__(256) void rotary_runs_kernel(const void* src, int s
   }
 }
 
+// The same runs with a wave a vector (widths up to 256), for runs whose vectors are divided by their root mean square
+// behind the turn (TurnRun.unit: x / sqrt(mean(x^2) + eps) over the vector's `width` entries): a lane holds the pairs
+// lane and lane + 64 of its vector, the squares are summed over the wave in one order, and the rows' results do not
+// depend on what else the step holds.  The grid is (rows, vectors of all runs / 4).
+__global__ __launch_bounds__(256) void rotary_runs_unit_kernel(const void* src, int src_dt, size_t ld_src, TurnRuns runs, const int* positions,
+                                                               const float* freq, float mag, float eps) {
+  const int t = blockIdx.x, lane = threadIdx.x & 63;
+  int vec = blockIdx.y * 4 + (threadIdx.x >> 6), r = 0;
+  while (r < runs.n && vec >= runs.run[r].n_vec) vec -= runs.run[r].n_vec, ++r;
+  if (r >= runs.n) return;      // (the whole wave)
+  const TurnRun& u = runs.run[r];
+  const float p = static_cast<float>(positions[t]);
+  const size_t a = static_cast<size_t>(t) * ld_src + u.src_off + static_cast<size_t>(vec) * u.width;
+  const size_t b = static_cast<size_t>(t) * u.ld_dst + u.dst_off + static_cast<size_t>(vec) * u.dst_stride;
+  float lo[2], hi[2];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int e = 2 * (lane + 64 * j);
+    lo[j] = e < u.width ? load_as(src, a + e, src_dt) : 0.f;
+    hi[j] = e + 1 < u.width ? load_as(src, a + e + 1, src_dt) : 0.f;
+    if (e + 1 < u.dims) {
+      const float ang = p * freq[e / 2];
+      const float c = cosf(ang) * mag, sn = sinf(ang) * mag;
+      const float x = lo[j], y = hi[j];
+      lo[j] = x * c - y * sn, hi[j] = y * c + x * sn;
+    }
+    ss = fmaf(lo[j], lo[j], ss);
+    ss = fmaf(hi[j], hi[j], ss);
+  }
+  float inv = 1.0f;
+  if (u.unit) inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(u.width) + eps);
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int e = 2 * (lane + 64 * j);
+    if (e < u.width) store_as(u.dst, b + e, u.dst_dt, lo[j] * inv);
+    if (e + 1 < u.width) store_as(u.dst, b + e + 1, u.dst_dt, hi[j] * inv);
+  }
+}
+
+// out[t, h * dv + d] = o[t, h * ldh + d] * sigmoid(g[t, h]) for d < dv: a gate per head on an attention's result, which
+// may lie in heads padded to ldh columns.
+__global__ __launch_bounds__(256) void head_gate_kernel(const void* o, int o_dt, size_t ldo, int head_stride, const float* g, size_t ldg,
+                                                        void* out, int out_dt, size_t ldout, int n_heads, int dv) {
+  const size_t t = blockIdx.x;
+  for (int e = threadIdx.x; e < n_heads * dv; e += 256) {
+    const int h = e / dv, d = e % dv;
+    const float v = load_as(o, t * ldo + static_cast<size_t>(h) * head_stride + d, o_dt);
+    store_as(out, t * ldout + e, out_dt, v * (1.0f / (1.0f + expf(-g[t * ldg + h]))));
+  }
+}
+
+// out[t, c] = a[t, c] * table[ids[t], off + c]: rows of a table picked by token, times rows of the step.
+__global__ __launch_bounds__(256) void rows_times_table_kernel(const void* a, int a_dt, size_t lda, const void* table, int t_dt, size_t ldt,
+                                                               int off, const int* ids, int n_rows, void* out, int out_dt, size_t ldo,
+                                                               int n) {
+  const size_t t = blockIdx.x;
+  const int id = ids[t];
+  for (int c = threadIdx.x; c < n; c += 256) {
+    // (an id outside the table gives NaN, never a neighbour's row; the host refuses it first)
+    const float e = (id >= 0 && id < n_rows) ? load_as(table, static_cast<size_t>(id) * ldt + off + c, t_dt) : __builtin_nanf("");
+    store_as(out, t * ldo + c, out_dt, load_as(a, t * lda + c, a_dt) * e);
+  }
+}
+
 // ---- activations of projections that feed a recurrence or a gate --------------------------------------------
-enum { ACT_SILU = 0, ACT_SIGMOID = 1, ACT_TANH = 2, ACT_EXP_NEG_EXP = 3, ACT_BOUNDED_SIGMOID = 4, ACT_EXP_NEG_SOFTPLUS = 5, ACT_XIELU = 6 };
+enum { ACT_SILU = 0, ACT_SIGMOID = 1, ACT_TANH = 2, ACT_EXP_NEG_EXP = 3, ACT_BOUNDED_SIGMOID = 4, ACT_EXP_NEG_SOFTPLUS = 5, ACT_XIELU = 6,
+       ACT_RELU2 = 7 };
 
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
 
@@ -304,6 +379,7 @@ __device__ __forceinline__ float activation(int kind, float z, float lower) {
     case ACT_SIGMOID: return sigmoid_f(z);
     case ACT_TANH: return tanhf(z);
     case ACT_EXP_NEG_EXP: return expf(-expf(z));
+    case ACT_RELU2: return fmaxf(z, 0.f) * fmaxf(z, 0.f);
     default: return lower + (1.0f - lower) * sigmoid_f(z);
   }
 }
@@ -720,6 +796,98 @@ __global__ __launch_bounds__(WAVES * 64) void gate_scan_kernel(const float* a, s
   if (live && wave == 0) *sp = S0;
 }
 
+// ---- a state per channel and state index with a decay of its own (the selective scan) -----------------------------
+// Over each request's rows in order, per channel c and state index n:
+//   dt = log(1 + e^(dt_in[t, c] + dt_bias[c]));  S[c, n] <- exp(dt A[c, n]) S[c, n] + dt x[t, c] B[t, n]
+//   y[t, c] = sum_n S[c, n] C[t, n] + D[c] x[t, c];  out[t, c] = y * silu(z[t, c])
+// A channel lies on 16 neighbouring lanes; lane l of them keeps the states n = l, l + 16, ... (PER of them) in registers
+// from a portion's first row to its last, and the sum over n is joined inside the row of 16 lanes, always in one order.
+// The rows are asked for TB at a time.  The same kernel for portions and for decoded tokens; a row's result depends on
+// the state before it alone, so how a prompt is cut changes nothing.
+struct SelectiveArgs {
+  const float *x, *dt, *dt_bias, *B, *C, *A, *D, *z;
+  size_t ldx, ldd, ldb, ldc, ldz;
+  float* state;
+  size_t slot_stride;
+  const int *row_start, *slots;
+  int inner, N;
+  void* out;
+  int out_dt;
+  size_t ldo;
+};
+
+template <int PER>
+__global__ __launch_bounds__(256) void selective_scan_kernel(SelectiveArgs a) {
+  constexpr int TB = PER >= 8 ? 1 : PER >= 4 ? 2 : 4;      // (rows in flight: what the registers hold beside the states)
+  const int s = blockIdx.y;
+  const int slot = a.slots[s];
+  if (slot < 0) return;      // (the whole workgroup: padding of a captured step)
+  const int row0 = a.row_start[s], row1 = a.row_start[s + 1];
+  if (row0 >= row1) return;
+  const int l = threadIdx.x & 15;
+  const int c = blockIdx.x * 16 + (threadIdx.x >> 4);
+  const bool live = c < a.inner;
+  const int cc = live ? c : a.inner - 1;
+  float rate[PER], S[PER];
+  int nn[PER];
+  float* sp = a.state + static_cast<size_t>(slot) * a.slot_stride + static_cast<size_t>(cc) * a.N;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int n = l + 16 * j;
+    const bool has = n < a.N;
+    nn[j] = has ? n : 0;
+    rate[j] = has ? a.A[static_cast<size_t>(cc) * a.N + n] : 0.f;      // (a place beyond N: decay 1 on a state of 0, B and C read as 0)
+    S[j] = has ? sp[n] : 0.f;
+  }
+  const float bias = a.dt_bias ? a.dt_bias[cc] : 0.f, skip = a.D ? a.D[cc] : 0.f;
+  float fx[TB], fd[TB], fz[TB], fb[TB][PER], fc[TB][PER];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      const size_t t = min(t0 + i, row1 - 1);
+      fx[i] = a.x[t * a.ldx + cc], fd[i] = a.dt[t * a.ldd + cc];
+      fz[i] = a.z ? a.z[t * a.ldz + cc] : 0.f;
+#pragma unroll
+      for (int j = 0; j < PER; ++j) fb[i][j] = a.B[t * a.ldb + nn[j]], fc[i][j] = a.C[t * a.ldc + nn[j]];
+    }
+  };
+  fetch(row0);
+  for (int t0 = row0; t0 < row1; t0 += TB) {
+    float x[TB], d[TB], z[TB], b[TB][PER], cm[TB][PER];
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      x[i] = fx[i], d[i] = fd[i], z[i] = fz[i];
+#pragma unroll
+      for (int j = 0; j < PER; ++j) b[i][j] = fb[i][j], cm[i][j] = fc[i][j];
+    }
+    if (t0 + TB < row1) fetch(t0 + TB);
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      if (t0 + i >= row1) break;
+      const float dt = softplus_f(d[i] + bias);
+      const float dx = dt * x[i];
+      float y = 0.f;
+#pragma unroll
+      for (int j = 0; j < PER; ++j) {
+        const bool has = l + 16 * j < a.N;
+        S[j] = fmaf(expf(dt * rate[j]), S[j], has ? dx * b[i][j] : 0.f);
+        y = fmaf(S[j], has ? cm[i][j] : 0.f, y);
+      }
+      y = group_reduce<16>(y, SumOp());
+      if (live && l == 0) {
+        y = fmaf(skip, x[i], y);
+        if (a.z) y *= z[i] / (1.0f + expf(-z[i]));
+        store_as(a.out, static_cast<size_t>(t0 + i) * a.ldo + c, a.out_dt, y);
+      }
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+      if (l + 16 * j < a.N) sp[l + 16 * j] = S[j];
+  }
+}
+
 // ---- queries and keys normed as whole vectors, keys and values to the cache -----------------------------------------
 // A row of z is [q: qw | k: kw].  q_out[t] = q / rms(q) * wq; the key that goes to the cache is k / rms(k) * wk, the value
 // k as it is (pools [page][key head][offset][dim] and [page][key head][dim][offset], the row's place from slot_map; a
@@ -944,12 +1112,12 @@ int dn_rmsnorm(const void* x, int x_dt, long long ldx, const float* weight, void
 }
 
 int dn_rmsnorm_add(const void* y, int y_dt, long long ldy, const float* weight, const float* scale, float mult, float* x, long long ldx,
-                   int T, int width, float eps, hipStream_t stream) {
+                   int T, int width, float eps, const float* gate, long long ldg, hipStream_t stream) {
   if (!float_kind(y_dt)) return DN_ERR_DTYPE;
-  if (T < 0 || width < 1) return DN_ERR_SHAPE;
+  if (T < 0 || width < 1 || (gate && ldg < width)) return DN_ERR_SHAPE;
   if (T == 0) return 0;
   hipLaunchKernelGGL(rmsnorm_add_kernel, dim3(T), dim3(256), 0, stream, y, y_dt, static_cast<size_t>(ldy), weight, scale, mult, x,
-                     static_cast<size_t>(ldx), width, eps);
+                     static_cast<size_t>(ldx), width, eps, gate, static_cast<size_t>(ldg));
   return dn_launch_status();
 }
 
@@ -1008,20 +1176,29 @@ int dn_conv_heads(const float* h, long long ldh, const float* w, const float* hi
 
 // runs: n x 9 numbers (dst, dst_dt, ld_dst, src_off, dst_off, dst_stride, n_vec, width, dims), n <= 3
 int dn_rotary_runs(const void* src, int src_dt, long long ld_src, const long long* runs, int n, const int* positions, const float* freq,
-                   int T, hipStream_t stream) {
+                   int T, float mag, long long unit_mask, float eps, hipStream_t stream) {
   if (!float_kind(src_dt) || n < 1 || n > 3) return n < 1 || n > 3 ? DN_ERR_SHAPE : DN_ERR_DTYPE;
   TurnRuns r{};
   r.n = n;
+  long long vectors = 0;
   for (int i = 0; i < n; ++i) {
     const long long* q = runs + 9 * i;
     r.run[i] = TurnRun{reinterpret_cast<void*>(q[0]), static_cast<int>(q[1]), static_cast<size_t>(q[2]), static_cast<int>(q[3]),
                        static_cast<int>(q[4]), static_cast<int>(q[5]), static_cast<int>(q[6]), static_cast<int>(q[7]),
-                       static_cast<int>(q[8])};
+                       static_cast<int>(q[8]), static_cast<int>((unit_mask >> i) & 1)};
     if (!float_kind(r.run[i].dst_dt)) return DN_ERR_DTYPE;
     if (r.run[i].dims % 2 != 0 || r.run[i].dims < 0 || r.run[i].dims > r.run[i].width || r.run[i].n_vec < 0) return DN_ERR_SHAPE;
+    if (unit_mask && r.run[i].width > 256) return DN_ERR_SHAPE;      // (a wave holds a vector of up to 256 numbers)
+    vectors += r.run[i].n_vec;
   }
   if (T == 0) return 0;
-  hipLaunchKernelGGL(rotary_runs_kernel, dim3(T), dim3(256), 0, stream, src, src_dt, static_cast<size_t>(ld_src), r, positions, freq);
+  if (unit_mask) {
+    if (vectors == 0 || (vectors + 3) / 4 > 65535) return vectors == 0 ? 0 : DN_ERR_SHAPE;
+    hipLaunchKernelGGL(rotary_runs_unit_kernel, dim3(T, (vectors + 3) / 4), dim3(256), 0, stream, src, src_dt, static_cast<size_t>(ld_src), r,
+                       positions, freq, mag, eps);
+    return dn_launch_status();
+  }
+  hipLaunchKernelGGL(rotary_runs_kernel, dim3(T), dim3(256), 0, stream, src, src_dt, static_cast<size_t>(ld_src), r, positions, freq, mag);
   return dn_launch_status();
 }
 
@@ -1046,20 +1223,20 @@ int dn_shift_mix(const void* h, int h_dt, const float* hist, const float* mu, in
 }
 
 int dn_rotary(const void* src, int src_dt, long long ld_src, int src_off, int src_stride, void* dst, int dst_dt, long long ld_dst,
-              int dst_off, int dst_stride, const int* positions, const float* freq, int T, int n_vec, int dims, int width,
+              int dst_off, int dst_stride, const int* positions, const float* freq, int T, int n_vec, int dims, int width, float mag,
               hipStream_t stream) {
   if (!float_kind(src_dt) || !float_kind(dst_dt)) return DN_ERR_DTYPE;
   if (dims % 2 != 0 || dims > width || dims < 0) return DN_ERR_SHAPE;
   if (T == 0 || n_vec == 0) return 0;
   hipLaunchKernelGGL(rotary_kernel, dim3(T), dim3(256), 0, stream, src, src_dt, static_cast<size_t>(ld_src), src_off, src_stride, dst,
-                     dst_dt, static_cast<size_t>(ld_dst), dst_off, dst_stride, positions, freq, n_vec, dims, width);
+                     dst_dt, static_cast<size_t>(ld_dst), dst_off, dst_stride, positions, freq, n_vec, dims, width, mag);
   return dn_launch_status();
 }
 
 int dn_activate(const float* x, long long ldx, const float* bias, const float* lower, int kind, void* out, int out_dt, long long ldo,
                 int T, int n, hipStream_t stream) {
   if (!float_kind(out_dt)) return DN_ERR_DTYPE;
-  if (kind < 0 || kind > ACT_XIELU || ((kind == ACT_XIELU || kind == ACT_EXP_NEG_SOFTPLUS) && !lower)) return DN_ERR_SHAPE;
+  if (kind < 0 || kind > ACT_RELU2 || ((kind == ACT_XIELU || kind == ACT_EXP_NEG_SOFTPLUS) && !lower)) return DN_ERR_SHAPE;
   if (T == 0) return 0;
   hipLaunchKernelGGL(activate_kernel, dim3(T), dim3(256), 0, stream, x, static_cast<size_t>(ldx), bias, lower, kind, out, out_dt,
                      static_cast<size_t>(ldo), n);
@@ -1214,6 +1391,46 @@ int dn_norm_pair_write(const float* z, long long ldz, int qw, int kw, const floa
   if (T == 0) return 0;
   hipLaunchKernelGGL(norm_pair_write_kernel, dim3(T), dim3(256), 0, stream, z, static_cast<size_t>(ldz), qw, kw, wq, wk, eps, q_out,
                      static_cast<size_t>(ldq), slot_map, k_pool, v_pool, dh, page_size, dt, write);
+  return dn_launch_status();
+}
+
+int dn_head_gate(const void* o, int o_dt, long long ldo, int head_stride, const float* g, long long ldg, void* out, int out_dt,
+                 long long ldout, int T, int n_heads, int dv, hipStream_t stream) {
+  if (!float_kind(o_dt) || !float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (n_heads < 1 || dv < 1 || head_stride < dv || ldg < n_heads) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(head_gate_kernel, dim3(T), dim3(256), 0, stream, o, o_dt, static_cast<size_t>(ldo), head_stride, g,
+                     static_cast<size_t>(ldg), out, out_dt, static_cast<size_t>(ldout), n_heads, dv);
+  return dn_launch_status();
+}
+
+int dn_rows_times_table(const void* a, int a_dt, long long lda, const void* table, int t_dt, long long ldt, int off, const int* ids,
+                        int n_rows, void* out, int out_dt, long long ldo, int T, int n, hipStream_t stream) {
+  if (!float_kind(a_dt) || !float_kind(t_dt) || !float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (n < 1 || off < 0 || off + n > ldt || n_rows < 1) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  hipLaunchKernelGGL(rows_times_table_kernel, dim3(T), dim3(256), 0, stream, a, a_dt, static_cast<size_t>(lda), table, t_dt,
+                     static_cast<size_t>(ldt), off, ids, n_rows, out, out_dt, static_cast<size_t>(ldo), n);
+  return dn_launch_status();
+}
+
+int dn_selective_scan(const float* x, long long ldx, const float* dt, long long ldd, const float* dt_bias, const float* B, long long ldb,
+                      const float* C, long long ldc, const float* A, const float* D, const float* z, long long ldz, float* state,
+                      long long slot_stride, const int* row_start, const int* slots, int S, int inner, int N, void* out, int out_dt,
+                      long long ldo, hipStream_t stream) {
+  if (!float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (inner < 1 || N < 1 || N > 256 || S > 65535 || slot_stride < static_cast<long long>(inner) * N) return DN_ERR_SHAPE;
+  if (S == 0) return 0;
+  const SelectiveArgs a{x, dt, dt_bias, B, C, A, D, z, static_cast<size_t>(ldx), static_cast<size_t>(ldd), static_cast<size_t>(ldb),
+                        static_cast<size_t>(ldc), static_cast<size_t>(ldz), state, static_cast<size_t>(slot_stride), row_start, slots,
+                        inner, N, out, out_dt, static_cast<size_t>(ldo)};
+  const dim3 grid((inner + 15) / 16, S);
+  const int per = (N + 15) / 16;
+  if (per <= 1) hipLaunchKernelGGL(selective_scan_kernel<1>, grid, dim3(256), 0, stream, a);
+  else if (per <= 2) hipLaunchKernelGGL(selective_scan_kernel<2>, grid, dim3(256), 0, stream, a);
+  else if (per <= 4) hipLaunchKernelGGL(selective_scan_kernel<4>, grid, dim3(256), 0, stream, a);
+  else if (per <= 8) hipLaunchKernelGGL(selective_scan_kernel<8>, grid, dim3(256), 0, stream, a);
+  else hipLaunchKernelGGL(selective_scan_kernel<16>, grid, dim3(256), 0, stream, a);
   return dn_launch_status();
 }
 

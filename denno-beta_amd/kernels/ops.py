@@ -130,15 +130,15 @@ def _declare(name, lib):
         "sequence": {
             "dn_rmsnorm": [P, I, c_longlong, P, P, I, c_longlong, P, I, I, F, P],
             "dn_concat_cast": [P, c_longlong, I, P, c_longlong, I, P, I, I, P],
-            "dn_rmsnorm_add": [P, I, c_longlong, P, P, F, P, c_longlong, I, I, F, P],
+            "dn_rmsnorm_add": [P, I, c_longlong, P, P, F, P, c_longlong, I, I, F, P, c_longlong, P],
             "dn_depth_mix": [P, c_longlong, I, P, P, c_longlong, P],
             "dn_unit_heads": [P, c_longlong, P, c_longlong, I, I, I, F, F, P],
             "dn_conv_rows": [P, c_longlong, P, P, P, P, P, I, I, I, I, I, I, P, I, c_longlong, c_longlong, P],
             "dn_history_update": [P, I, c_longlong, P, P, P, I, I, I, c_longlong, P],
             "dn_conv_heads": [P, c_longlong, P, P, P, P, I, I, I, I, I, I, F, F, F, I, I, P, c_longlong, c_longlong, P],
-            "dn_rotary_runs": [P, I, c_longlong, P, I, P, P, I, P],
+            "dn_rotary_runs": [P, I, c_longlong, P, I, P, P, I, F, c_longlong, F, P],
             "dn_shift_mix": [P, I, P, P, I, P, P, I, I, I, P, I, c_longlong, P],
-            "dn_rotary": [P, I, c_longlong, I, I, P, I, c_longlong, I, I, P, P, I, I, I, I, P],
+            "dn_rotary": [P, I, c_longlong, I, I, P, I, c_longlong, I, I, P, P, I, I, I, I, F, P],
             "dn_activate": [P, c_longlong, P, P, I, P, I, c_longlong, I, I, P],
             "dn_gated": [P, I, c_longlong, P, c_longlong, I, P, I, c_longlong, I, I, P],
             "dn_state_scan": [P, c_longlong, P, c_longlong, P, c_longlong, P, c_longlong, P, P, c_longlong, P, I, P, c_longlong, P, P,
@@ -149,10 +149,14 @@ def _declare(name, lib):
             "dn_streams_read": [P, c_longlong, I, P, P, F, P, I, c_longlong, P, I, I, P],
             "dn_streams_write": [P, c_longlong, I, P, P, P, c_longlong, P, c_longlong, P, P, F, P, P, F, P, I, c_longlong, I, I, P],
             "dn_norm_pair_write": [P, c_longlong, I, I, P, P, F, P, c_longlong, P, P, P, I, I, I, I, I, I, P],
+            "dn_head_gate": [P, I, c_longlong, I, P, c_longlong, P, I, c_longlong, I, I, I, P],
+            "dn_rows_times_table": [P, I, c_longlong, P, I, c_longlong, I, P, I, P, I, c_longlong, I, I, P],
+            "dn_selective_scan": [P, c_longlong, P, c_longlong, P, P, c_longlong, P, c_longlong, P, P, P, c_longlong, P, c_longlong,
+                                  P, P, I, I, I, P, I, c_longlong, P],
         },
         "grouped": {
             "dn_heads_linear": [P, I, c_longlong, I, I, P, I, P, I, c_longlong, I, I, I, I, I, I, P],
-            "dn_moe_route": [P, c_longlong, P, I, I, I, I, I, P, P, P],
+            "dn_moe_route": [P, c_longlong, P, I, I, I, I, I, P, P, I, I, F, P],
             "dn_moe_plan": [P, I, I, P, P, P],
             "dn_moe_up": [P, I, c_longlong, P, P, I, I, I, P, P, I, I, I, F, F, I, P, P, I, I, P],
             "dn_moe_down": [P, I, P, P, I, I, P, I, I, I, P, I, P],
@@ -957,7 +961,7 @@ def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None, n
 
 
 # -- layers that carry more than keys and values from token to token (csrc/kernels/sequence.hip) -----------------------
-ACTIVATIONS = {"silu": 0, "sigmoid": 1, "tanh": 2, "exp_neg_exp": 3, "bounded_sigmoid": 4, "exp_neg_softplus": 5, "xielu": 6}
+ACTIVATIONS = {"silu": 0, "sigmoid": 1, "tanh": 2, "exp_neg_exp": 3, "bounded_sigmoid": 4, "exp_neg_softplus": 5, "xielu": 6, "relu2": 7}
 
 
 def _f32vec(t, name, n=None):
@@ -1000,15 +1004,20 @@ def rmsnorm(x, weight, eps, out, rows=None):
     return out
 
 
-def rmsnorm_add(y, weight, scale, mult, eps, x):
+def rmsnorm_add(y, weight, scale, mult, eps, x, gate=None):
     """x[t, :] += mult * (y[t, :] / sqrt(mean(y[t, :]^2) + eps) * weight) * scale; weight and scale: 32-bit vectors or None;
-    x: 32-bit rows (the stream), changed in place; statistics in 32-bit."""
+    x: 32-bit rows (the stream), changed in place; statistics in 32-bit.  gate: 32-bit [T, width] (columns of wider rows):
+    y is y * sigmoid(gate) first, under the norm too."""
     _dev(y, "y", _FLOATS, 2), _dev(x, "x", (torch.float32,), 2)
     T, width = y.shape
     _need(tuple(x.shape) == (T, width), "rmsnorm_add: shapes")
     _f32vec(weight, "weight", width), _f32vec(scale, "scale", width)
+    if gate is not None:
+        _dev(gate, "gate", (torch.float32,), 2)
+        _need(tuple(gate.shape) == (T, width), "rmsnorm_add: gate")
     _ok(_lib("sequence").dn_rmsnorm_add(y.data_ptr(), _CODE[y.dtype], _rows(y, "y"), _ptr(weight), _ptr(scale), float(mult),
-                                        x.data_ptr(), _rows(x, "x"), T, width, float(eps), _stream()), "rmsnorm_add")
+                                        x.data_ptr(), _rows(x, "x"), T, width, float(eps), _ptr(gate),
+                                        _rows(gate, "gate") if gate is not None else 0, _stream()), "rmsnorm_add")
     return x
 
 
@@ -1097,17 +1106,22 @@ def conv_heads(h, w, hist, row_start, slots, out, n_unit, unit_dim, n_first, sca
     return out
 
 
-def rotary_runs(src, positions, freq, runs):
+def rotary_runs(src, positions, freq, runs, mag=1.0, unit=None, eps=0.0):
     """Up to three runs of vectors of src's rows in one launch.  runs: [(dst, src_off, n_vec, width, dims, dst_off, dst_stride)]:
     the n_vec vectors of `width` numbers that lie side by side from column src_off go to columns dst_off + n * dst_stride of
-    dst, their first `dims` entries turned in pairs by positions[t] * freq[i] (dims 0: only moved); as `rotary` does."""
+    dst, their first `dims` entries turned in pairs by positions[t] * freq[i] (dims 0: only moved); as `rotary` does.
+    mag multiplies cos and sin.  unit: a flag per run: the run's vectors are divided by their root mean square behind the
+    turn, x / sqrt(mean(x^2) + eps) over their `width` entries (vectors of up to 256 numbers then, in every run)."""
     _dev(src, "src", _FLOATS, 2), _dev(positions, "positions", _I32, 1)
     T = src.shape[0]
     _need(1 <= len(runs) <= 3 and positions.is_contiguous() and positions.shape[0] == T, "rotary_runs: runs or rows")
+    unit = [False] * len(runs) if unit is None else [bool(u) for u in unit]
+    _need(len(unit) == len(runs), "rotary_runs: a unit flag per run")
     table, most = [], 0
     for dst, src_off, n_vec, width, dims, dst_off, dst_stride in runs:
         _dev(dst, "dst", _FLOATS, 2)
         _need(dst.shape[0] == T and dims % 2 == 0 and 0 <= dims <= width and n_vec >= 0, "rotary_runs: a run's sizes")
+        _need(not any(unit) or width <= 256, lambda: f"rotary_runs: vectors of {width} numbers; with a norm behind the turn up to 256")
         if n_vec:
             _need(src_off >= 0 and src_off + n_vec * width <= src.shape[1] and dst_off >= 0
                   and dst_off + (n_vec - 1) * dst_stride + width <= dst.shape[1], "rotary_runs: vectors outside their rows")
@@ -1117,8 +1131,9 @@ def rotary_runs(src, positions, freq, runs):
     _need(freq.numel() >= most // 2 and all(r[4] in (0, most) for r in runs), "rotary_runs: one table of frequencies for the turned runs")
     import ctypes
     arr = (ctypes.c_longlong * len(table))(*table)
+    mask = sum(1 << i for i, u in enumerate(unit) if u)
     _ok(_lib("sequence").dn_rotary_runs(src.data_ptr(), _CODE[src.dtype], _rows(src, "src"), arr, len(runs), positions.data_ptr(),
-                                        freq.data_ptr(), T, _stream()), "rotary_runs")
+                                        freq.data_ptr(), T, float(mag), mask, float(eps), _stream()), "rotary_runs")
 
 
 def shift_mix(h, hist, mu, row_start, slots, out):
@@ -1135,10 +1150,10 @@ def shift_mix(h, hist, mu, row_start, slots, out):
     return out
 
 
-def rotary(src, dst, positions, freq, n_vec, dims, width, src_off=0, src_stride=None, dst_off=0, dst_stride=None):
+def rotary(src, dst, positions, freq, n_vec, dims, width, src_off=0, src_stride=None, dst_off=0, dst_stride=None, mag=1.0):
     """Vector n (n < n_vec) of row t, `width` wide, starts at column src_off + n * src_stride of src; of its first `dims`
-    entries, 2i and 2i + 1 are turned by positions[t] * freq[i] (32-bit angles), the rest pass; it goes to column
-    dst_off + n * dst_stride of dst (which may be src)."""
+    entries, 2i and 2i + 1 are turned by positions[t] * freq[i] (32-bit angles; cos and sin times `mag`), the rest pass; it
+    goes to column dst_off + n * dst_stride of dst (which may be src)."""
     _dev(src, "src", _FLOATS, 2), _dev(dst, "dst", _FLOATS, 2), _dev(positions, "positions", _I32, 1)
     T = src.shape[0]
     src_stride = width if src_stride is None else src_stride
@@ -1151,14 +1166,15 @@ def rotary(src, dst, positions, freq, n_vec, dims, width, src_off=0, src_stride=
               and dst_off >= 0 and dst_off + (n_vec - 1) * dst_stride + width <= dst.shape[1], "rotary: vectors outside their rows")
     _ok(_lib("sequence").dn_rotary(src.data_ptr(), _CODE[src.dtype], _rows(src, "src"), src_off, src_stride, dst.data_ptr(),
                                    _CODE[dst.dtype], _rows(dst, "dst"), dst_off, dst_stride, positions.data_ptr(), freq.data_ptr(),
-                                   T, n_vec, dims, width, _stream()), "rotary")
+                                   T, n_vec, dims, width, float(mag), _stream()), "rotary")
     return dst
 
 
 def activate(x, kind, out, bias=None, lower=None):
     """out = act(x + bias): "silu", "sigmoid", "tanh", "exp_neg_exp" (exp(-exp(z))), "bounded_sigmoid"
     (lower + (1 - lower) * sigmoid(z)), "exp_neg_softplus" (exp(-lower * log(1 + e^z)), lower a rate per column), "xielu"
-    (z > 0: a z^2 + z / 2, else b (e^z - 1 - z) + z / 2, with lower = (a, b), two numbers).  x 32-bit; out may be x."""
+    (z > 0: a z^2 + z / 2, else b (e^z - 1 - z) + z / 2, with lower = (a, b), two numbers), "relu2" (max(z, 0)^2).  x 32-bit; out
+    may be x."""
     _dev(x, "x", (torch.float32,), 2), _dev(out, "out", _FLOATS, 2)
     T, n = x.shape
     _need(tuple(out.shape) == (T, n), "activate: shapes")
@@ -1280,6 +1296,56 @@ def gate_scan(a, b, g, bias_a, bias_b, state, row_start, slots, out):
     return out
 
 
+def head_gate(o, gate, n_heads, dv, out, head_stride=None):
+    """out[t, h * dv + d] = o[t, h * head_stride + d] * sigmoid(gate[t, h]) for d < dv: a gate per head on heads that may be
+    padded to head_stride columns (None: dv).  gate: 32-bit [T, n_heads] (columns of wider rows)."""
+    _dev(o, "o", _FLOATS, 2), _dev(gate, "gate", (torch.float32,), 2), _dev(out, "out", _FLOATS, 2)
+    T = o.shape[0]
+    hs = dv if head_stride is None else head_stride
+    _need(hs >= dv >= 1 and n_heads >= 1 and o.shape[1] >= (n_heads - 1) * hs + dv and tuple(gate.shape) == (T, n_heads)
+          and tuple(out.shape) == (T, n_heads * dv), "head_gate: shapes")
+    _ok(_lib("sequence").dn_head_gate(o.data_ptr(), _CODE[o.dtype], _rows(o, "o"), hs, gate.data_ptr(), _rows(gate, "gate"),
+                                      out.data_ptr(), _CODE[out.dtype], _rows(out, "out"), T, n_heads, dv, _stream()), "head_gate")
+    return out
+
+
+def rows_times_table(a, table, ids, off, out):
+    """out[t, c] = a[t, c] * table[ids[t], off + c] for the columns of a: rows of a table picked by an index per row."""
+    _dev(a, "a", _FLOATS, 2), _dev(table, "table", _FLOATS, 2), _dev(ids, "ids", _I32, 1), _dev(out, "out", _FLOATS, 2)
+    T, n = a.shape
+    _need(tuple(out.shape) == (T, n) and ids.is_contiguous() and ids.shape[0] == T and off >= 0 and off + n <= table.shape[1],
+          "rows_times_table: shapes")
+    _ok(_lib("sequence").dn_rows_times_table(a.data_ptr(), _CODE[a.dtype], _rows(a, "a"), table.data_ptr(), _CODE[table.dtype],
+                                             _rows(table, "table"), off, ids.data_ptr(), table.shape[0], out.data_ptr(),
+                                             _CODE[out.dtype], _rows(out, "out"), T, n, _stream()), "rows_times_table")
+    return out
+
+
+def selective_scan(x, dt, dt_bias, B, C, A, D, z, state, row_start, slots, out):
+    """A state per channel c and state index n with a decay of its own, over each request's rows in order:
+      step = log(1 + e^(dt[t, c] + dt_bias[c]));  S[c, n] <- exp(step * A[c, n]) S[c, n] + step * x[t, c] * B[t, n]
+      y[t, c] = sum_n S[c, n] C[t, n] + D[c] x[t, c];  out[t, c] = y * silu(z[t, c])      (z None: y as it is)
+    x, dt, z: 32-bit [T, inner]; B, C: 32-bit [T, N] (all may be columns of wider rows); A: 32-bit [inner, N]; dt_bias, D:
+    32-bit [inner] or None; state: 32-bit [slots, inner * N], read and written at the requests' slots; out [T, inner]."""
+    for t, name in ((x, "x"), (dt, "dt"), (B, "B"), (C, "C")) + (((z, "z"),) if z is not None else ()):
+        _dev(t, name, (torch.float32,), 2)
+    _dev(out, "out", _FLOATS, 2), _dev(A, "A", (torch.float32,), 2)
+    T, inner = x.shape
+    N = B.shape[1]
+    S = _request_tables(row_start, slots, "selective_scan")
+    _need(tuple(dt.shape) == (T, inner) and tuple(B.shape) == (T, N) and tuple(C.shape) == (T, N) and tuple(out.shape) == (T, inner)
+          and (z is None or tuple(z.shape) == (T, inner)) and tuple(A.shape) == (inner, N) and A.is_contiguous(), "selective_scan: shapes")
+    _need(1 <= N <= 256, lambda: f"selective_scan: {N} states a channel; the kernel keeps up to 256 on a channel's lanes")
+    _f32vec(dt_bias, "dt_bias", inner), _f32vec(D, "D", inner)
+    stride = _history(state, inner * N, "selective_scan")
+    _ok(_lib("sequence").dn_selective_scan(x.data_ptr(), _rows(x, "x"), dt.data_ptr(), _rows(dt, "dt"), _ptr(dt_bias), B.data_ptr(),
+                                           _rows(B, "B"), C.data_ptr(), _rows(C, "C"), A.data_ptr(), _ptr(D), _ptr(z),
+                                           _rows(z, "z") if z is not None else 0, state.data_ptr(), stride, row_start.data_ptr(),
+                                           slots.data_ptr(), S, inner, N, out.data_ptr(), _CODE[out.dtype], _rows(out, "out"),
+                                           _stream()), "selective_scan")
+    return out
+
+
 STREAMS_MAX = 8
 
 
@@ -1373,19 +1439,23 @@ def heads_linear(a, w, out, a_off=0, a_stride=None, o_off=0, o_stride=None):
     return out
 
 
-def moe_route(z, correction, top, ids, wts, score="softmax", renorm=True, n_experts=None):
+def moe_route(z, correction, top, ids, wts, score="softmax", renorm=True, n_experts=None, groups=1, keep=1, scale=1.0):
     """Per row: s = softmax(z) over the experts, or (score "sigmoid") each expert's own 1 / (1 + e^-z); the `top` experts with
     the largest s + correction (the lower index wins a tie) go to ids [T, top]; wts [T, top] gets their s divided by the sum
-    of the chosen s (+ 1e-20), or (renorm False) their s as it is.  n_experts: the first columns of z that are experts
-    (None: all of them)."""
+    of the chosen s (+ 1e-20), or (renorm False) their s as it is, times `scale`.  n_experts: the first columns of z that are
+    experts (None: all of them).  groups > 1: the experts are that many equal runs of neighbours, a group's score is the sum
+    of its two largest s + correction, and only experts of the `keep` best groups can be chosen."""
     _dev(z, "z", (torch.float32,), 2), _dev(ids, "ids", _I32, 2), _dev(wts, "wts", (torch.float32,), 2)
     T = z.shape[0]
     E = z.shape[1] if n_experts is None else n_experts
     _need(ids.is_contiguous() and wts.is_contiguous() and tuple(ids.shape) == (T, top) and E <= z.shape[1]
           and tuple(wts.shape) == (T, top) and 1 <= top <= E and score in ("softmax", "sigmoid"), "moe_route: shapes")
+    _need(groups >= 1 and E % groups == 0 and 1 <= keep <= groups and top <= keep * (E // groups),
+          lambda: f"moe_route: {E} experts in {groups} groups of which {keep} are kept, for {top} choices")
     _f32vec(correction, "correction", E)
     _ok(_lib("grouped").dn_moe_route(z.data_ptr(), _rows(z, "z"), _ptr(correction), T, E, top, int(score == "sigmoid"),
-                                     int(bool(renorm)), ids.data_ptr(), wts.data_ptr(), _stream()), "moe_route")
+                                     int(bool(renorm)), ids.data_ptr(), wts.data_ptr(), int(groups), int(keep), float(scale),
+                                     _stream()), "moe_route")
 
 
 def moe_plan(ids, n_experts, offsets, order):
@@ -1408,29 +1478,34 @@ def moe_up(h, order, offsets, top, w_gate, w_up, limit, alpha, y, dims=None, kin
     """For place p of expert e, the row t = order[p] // top: kind "clamped": g = min(w_gate[e] h[t], limit), u = clamp(w_up[e]
     h[t], -limit, limit), y[p] = g * sigmoid(alpha * g) * (u + 1); kind "silu": the expert reads s h[t] with s =
     in_scale[order[p]] (32-bit [T * top]; None: 1), y[p] = silu(w_gate[e] s h[t]) * (w_up[e] s h[t]), the factor applied to
-    the 32-bit sums.  w_gate, w_up: [experts, ff, width]; y [T * top, ff].
+    the 32-bit sums; kind "relu2": an expert without a gate (w_gate None), y[p] = max(w_up[e] s h[t], 0)^2.
+    w_gate, w_up: [experts, ff, width]; y [T * top, ff].
     dims = (experts, ff, width): w_gate and w_up are PackedMatrix of the stacked [experts * ff, width] (experts_packable)."""
     _dev(h, "h", _FLOATS, 2), _dev(y, "y", _FLOATS, 2)
     n = order.shape[0]
+    _need(kind in ("clamped", "silu", "relu2") and (w_gate is None) == (kind == "relu2"), "moe_up: kind, or a gate that it does not have")
     if dims is not None:
         E, ff, width = dims
-        _need(isinstance(w_gate, PackedMatrix) and isinstance(w_up, PackedMatrix) and tuple(w_gate.shape) == (E * ff, width)
-              and tuple(w_up.shape) == (E * ff, width) and experts_packable(E, ff, width), "moe_up: packed weights")
+        _need(all(w is None or (isinstance(w, PackedMatrix) and tuple(w.shape) == (E * ff, width)) for w in (w_gate, w_up))
+              and experts_packable(E, ff, width), "moe_up: packed weights")
         wdt = torch.bfloat16
     else:
-        _dev(w_gate, "w_gate", _FLOATS, 3), _dev(w_up, "w_up", (w_gate.dtype,), 3)
-        E, ff, width = w_gate.shape
-        _need(w_gate.is_contiguous() and w_up.is_contiguous() and tuple(w_up.shape) == (E, ff, width), "moe_up: weights")
-        wdt = w_gate.dtype
+        _dev(w_up, "w_up", _FLOATS, 3)
+        E, ff, width = w_up.shape
+        _need(w_up.is_contiguous(), "moe_up: weights")
+        if w_gate is not None:
+            _dev(w_gate, "w_gate", (w_up.dtype,), 3)
+            _need(w_gate.is_contiguous() and tuple(w_gate.shape) == (E, ff, width), "moe_up: weights")
+        wdt = w_up.dtype
     _need(h.shape[1] == width and y.is_contiguous() and tuple(y.shape) == (n, ff) and offsets.shape[0] == E + 1
-          and n == h.shape[0] * top and kind in ("clamped", "silu"), "moe_up: shapes")
+          and n == h.shape[0] * top, "moe_up: shapes")
     if in_scale is not None:
         _dev(in_scale, "in_scale", (torch.float32,))
-        _need(in_scale.is_contiguous() and in_scale.numel() == n and kind == "silu", "moe_up: in_scale")
+        _need(in_scale.is_contiguous() and in_scale.numel() == n and kind != "clamped", "moe_up: in_scale")
     _ok(_lib("grouped").dn_moe_up(h.data_ptr(), _CODE[h.dtype], _rows(h, "h"), order.data_ptr(), offsets.data_ptr(), E, top, n,
-                                  w_gate.data_ptr(), w_up.data_ptr(), _CODE[wdt], ff, width, float(limit), float(alpha),
-                                  int(kind == "silu"), _ptr(in_scale), y.data_ptr(), _CODE[y.dtype], int(dims is not None),
-                                  _stream()), "moe_up")
+                                  w_gate.data_ptr() if w_gate is not None else 0, w_up.data_ptr(), _CODE[wdt], ff, width, float(limit),
+                                  float(alpha), {"clamped": 0, "silu": 1, "relu2": 2}[kind], _ptr(in_scale), y.data_ptr(),
+                                  _CODE[y.dtype], int(dims is not None), _stream()), "moe_up")
 
 
 def moe_down(y, order, offsets, w_down, out, dims=None):

@@ -1,2 +1,2 @@
 """Architectures the framework ships.  Importing a module registers it."""
-from . import dogalorn, gpt2, pafivik, ridopel   # noqa: F401
+from . import dogalorn, gpt2, nigilorn, pafivik, ridopel   # noqa: F401

@@ -13,6 +13,8 @@ Kinds of part and their registries:
   input filter     FILTERS         forward(h, ctx, cache) -> what the mixer reads ; cache_spec()
   connector        CONNECTORS      read(xs, norm, out_dtype) -> what a sublayer reads of several copies of the stream;
                                    write(xs, y): the copies anew from a sublayer's result
+  result gate      GATES           logits(h) -> 32-bit [T, width]: what a sublayer returns is multiplied by their sigmoid
+  token input      TOKEN_INPUTS    forward(x, ctx): adds to the stream what the rows' own tokens pick from a table
   position code    POSITIONS       table() for the embedding stage, rotate(q, k, ctx) for mixers
   arrangement      ARRANGEMENTS    SLOTS names its parts and their kinds; forward(x, ctx, caches, runtime): how
                                    norms, mixers and feed-forwards stand in a block
@@ -81,6 +83,8 @@ class Runtime:
     # next reads it first (set by the model), and the rows that the block before has read for this one in its last write's kernel
     next_read: Optional[tuple] = None
     stream_rows: Optional[torch.Tensor] = None
+    # the model's further tables by name (DecoderSpec.tables), for parts that pick rows of them (set by the model)
+    tables: Dict[str, torch.Tensor] = field(default_factory=dict)
 
 
 class Part:
@@ -210,5 +214,8 @@ POSITIONS = Registry("position encoding")
 ARRANGEMENTS = Registry("block arrangement")
 FILTERS = Registry("input filter")
 CONNECTORS = Registry("connector")
+GATES = Registry("result gate")
+TOKEN_INPUTS = Registry("token input")
 # the kinds that an arrangement's SLOTS may name
-KINDS = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "filter": FILTERS, "connector": CONNECTORS}
+KINDS = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "filter": FILTERS, "connector": CONNECTORS,
+         "gate": GATES, "token_input": TOKEN_INPUTS}

@@ -184,6 +184,37 @@ class SandwichBlock:
             self.post2.add_into(self._result(self.ffn, x, h, ctx), x)
 
 
+@ARRANGEMENTS.register("gated_sandwich")
+class GatedSandwichBlock(SandwichBlock):
+    """The sandwich with a gate on each sublayer's result and a token input at the end: with h = norm1(x),
+    x += post1(mixer(h) * sigmoid(gate1(h))); with h = norm2(x), x += post2(ffn(h) * sigmoid(gate2(h))); then the token
+    input adds what the rows' tokens pick (parts.token_inputs).  A gate reads the rows its sublayer read; the
+    multiplication runs inside the kernel of the norm behind.  Gates and token input may be "none"; a block whose
+    feed-forward is "none" goes from the mixer straight to the token input."""
+
+    SLOTS = {"norm1": "norm", "mixer": "mixer", "gate1": "gate", "post1": "norm", "norm2": "norm", "ffn": "feed_forward",
+             "gate2": "gate", "post2": "norm", "side": "token_input"}
+
+    def __init__(self, norm1, mixer, gate1, post1, norm2, ffn, gate2, post2, side):
+        super().__init__(norm1, mixer, post1, norm2, ffn, post2)
+        self.gate1, self.gate2, self.side = gate1, gate2, side
+        self.has_side = not getattr(side, "absent", False)
+
+    def parts(self):
+        return ([self.norm1, self.mixer, self.gate1, self.post1]
+                + ([self.norm2, self.ffn, self.gate2, self.post2] if self.has_ffn else []) + ([self.side] if self.has_side else []))
+
+    def forward(self, x, ctx, caches, runtime):
+        runtime.stream_stats = None
+        h = self.norm1.forward(x, runtime.act_dtype)
+        self.post1.add_into(self._result(self.mixer, x, h, ctx, caches[0]), x, gate=self.gate1.logits(h))
+        if self.has_ffn:
+            h = self.norm2.forward(x, runtime.act_dtype)
+            self.post2.add_into(self._result(self.ffn, x, h, ctx), x, gate=self.gate2.logits(h))
+        if self.has_side:
+            self.side.forward(x, ctx)
+
+
 @ARRANGEMENTS.register("multi_stream")
 class MultiStreamBlock:
     """The stream is several copies (DecoderSpec.streams).  For each sublayer f (the mixer, then the feed-forward) with its

@@ -80,6 +80,38 @@ class DenseMLP(Part):
         self.down(f, residual=accumulate_into, stats=stats, deferred=deferred)
 
 
+@FEED_FORWARDS.register("gated_mlp")
+class GatedMLP(Part):
+    """W_down (act(W_gate h) * (W_up h)), act "silu"; no biases.  Gate and up are one product whose 32-bit result the
+    activation reads."""
+    graph_safe = True
+    returns_rows = True
+    libraries = ("sequence",)
+
+    def __init__(self, width: int, inner: int, gate_weight: str, up_weight: str, down_weight: str, activation: str = "silu"):
+        if activation != "silu":
+            raise ValueError(f"gated_mlp: activation {activation!r}; known: ['silu']")
+        self.width, self.inner, self.activation = width, inner, activation
+        self.up = Linear(width, 2 * inner, gate_weight + "+up", None, init_std=width ** -0.5,
+                         weight_sources=((gate_weight, inner), (up_weight, inner)))
+        self.down = Linear(inner, width, down_weight, None, init_std=inner ** -0.5)
+
+    def param_specs(self):
+        return self.up.param_specs() + self.down.param_specs()
+
+    def bind(self, tensors, runtime):
+        super().bind(tensors, runtime)
+        self.up.bind(tensors), self.down.bind(tensors)
+
+    def forward(self, h, ctx, accumulate_into):
+        n = self.inner
+        gu = self.up(h, out_dtype=F32)
+        f = ops.gated(gu[:, n:], gu[:, :n], self.activation, torch.empty((h.shape[0], n), dtype=self.runtime.act_dtype, device=h.device))
+        if accumulate_into is None:
+            return self.down(f, out_dtype=F32)
+        self.down(f, residual=accumulate_into)
+
+
 @FEED_FORWARDS.register("none")
 class NoFeedForward(Part):
     """A block without a feed-forward: nothing is added to the stream (and the block does not run the norm before it)."""
@@ -104,22 +136,31 @@ class RoutedExperts(Part):
     What an architecture may choose otherwise: score "sigmoid" (each expert's own 1 / (1 + e^-z)); renorm False (the
     weights are the chosen scores as they are); weigh "input" (a weight multiplies what the expert reads, not what it
     returns); act "silu" (an expert is W_down (silu(W_gate h) * (W_up h)), nothing clamped; limit and alpha are then not
-    used); shared: an expert of the same form that every token uses, dict(inner, gate, up, down, token_gate): its result is
-    added, times sigmoid(w . h) with w the vector `token_gate` (a name, or None: as it is)."""
+    used), act "relu2" (an expert without a gate, W_down max(W_up h, 0)^2; `gate` is then None, also the shared expert's);
+    shared: an expert of the same form that every token uses, dict(inner, gate, up, down, token_gate): its result is
+    added, times sigmoid(w . h) with w the vector `token_gate` (a name, or None: as it is); groups and keep: the experts are
+    `groups` equal runs of neighbours, a group's score is the sum of its two largest s + correction, and only the experts
+    of the `keep` best groups can be chosen; route_scale multiplies the weights."""
     graph_safe = True
     returns_rows = True
     libraries = ("grouped", "sequence")
 
     def __init__(self, width: int, inner: int, n_experts: int, top: int, router: str, correction, gate: str, up: str, down: str,
                  limit: float = 0.0, alpha: float = 1.0, score: str = "softmax", renorm: bool = True, weigh: str = "output",
-                 act: str = "clamped", shared=None):
+                 act: str = "clamped", shared=None, groups: int = 1, keep: int = 1, route_scale: float = 1.0):
         """gate, up, down: tensor names with {e} for the expert's number; correction: a name or None."""
         if not 1 <= top <= n_experts:
             raise ValueError(f"routed_experts: {top} of {n_experts} experts")
-        if score not in ("softmax", "sigmoid") or weigh not in ("output", "input") or act not in ("clamped", "silu"):
+        if score not in ("softmax", "sigmoid") or weigh not in ("output", "input") or act not in ("clamped", "silu", "relu2"):
             raise ValueError(f"routed_experts: score {score!r}, weigh {weigh!r}, act {act!r}")
         if weigh == "input" and act != "silu":
             raise ValueError("routed_experts: a weight on what the expert reads goes with act 'silu'")
+        if (act == "relu2") != (gate is None):
+            raise ValueError("routed_experts: act 'relu2' is an expert without a gate matrix, and only that one")
+        if groups < 1 or n_experts % groups != 0 or not 1 <= keep <= groups or top > keep * (n_experts // groups):
+            raise ValueError(f"routed_experts: {n_experts} experts in {groups} groups of which {keep} are kept, for {top} choices")
+        self.groups, self.keep, self.route_scale = int(groups), int(keep), float(route_scale)
+        self.gated = gate is not None
         self.width, self.inner, self.n_experts, self.top = width, inner, n_experts, top
         self.limit, self.alpha = float(limit), float(alpha)
         self.score, self.renorm, self.weigh, self.act = score, bool(renorm), weigh, act
@@ -135,8 +176,11 @@ class RoutedExperts(Part):
             self.router = Linear(width, n_experts, router, None)
         if self.shared:
             sh = self.shared
-            self.shared_up = Linear(width, 2 * sh["inner"], sh["gate"] + "+up", None, init_std=width ** -0.5,
-                                    weight_sources=((sh["gate"], sh["inner"]), (sh["up"], sh["inner"])))
+            if self.gated:
+                self.shared_up = Linear(width, 2 * sh["inner"], sh["gate"] + "+up", None, init_std=width ** -0.5,
+                                        weight_sources=((sh["gate"], sh["inner"]), (sh["up"], sh["inner"])))
+            else:
+                self.shared_up = Linear(width, sh["inner"], sh["up"], None, init_std=width ** -0.5)
             self.shared_down = Linear(sh["inner"], width, sh["down"], None)
 
     def _stacked(self, which):
@@ -147,7 +191,7 @@ class RoutedExperts(Part):
                          sources=tuple((t.format(e=e), rows) for e in range(E)), concat_dim=0)
 
     def param_specs(self):
-        specs = self.router.param_specs() + [self._stacked(w) for w in ("gate", "up", "down")]
+        specs = self.router.param_specs() + [self._stacked(w) for w in (("gate", "up", "down") if self.gated else ("up", "down"))]
         if self.correction_name:
             specs.append(ParamSpec(self.correction_name, (self.n_experts,), "vector", ("normal", 0.0, 0.02)))
         if self.shared:
@@ -160,22 +204,23 @@ class RoutedExperts(Part):
         if self.shared:
             self.shared_up.bind(tensors), self.shared_down.bind(tensors)
         E = self.n_experts
-        self.w_gate = tensors[self.templates["gate"].format(e="*")].view(E, self.inner, self.width)
+        self.w_gate = tensors[self.templates["gate"].format(e="*")].view(E, self.inner, self.width) if self.gated else None
         self.w_up = tensors[self.templates["up"].format(e="*")].view(E, self.inner, self.width)
         self.w_down = tensors[self.templates["down"].format(e="*")].view(E, self.width, self.inner)
         self.correction = tensors[self.correction_name] if self.correction_name else None
         # bfloat16 experts on the GPU are held packed for the matrix cores, the stack as one matrix, where an expert's
         # rows start at a block's border (the rows they came from are not kept)
         self.up_dims = self.down_dims = None
-        if self.w_gate.dtype == torch.bfloat16 and self.w_gate.is_cuda:
+        if self.w_up.dtype == torch.bfloat16 and self.w_up.is_cuda:
             if ops.experts_packable(E, self.inner, self.width):
-                self.w_gate = ops.pack_matrix(self.w_gate.view(E * self.inner, self.width))
+                if self.gated:
+                    self.w_gate = ops.pack_matrix(self.w_gate.view(E * self.inner, self.width))
                 self.w_up = ops.pack_matrix(self.w_up.view(E * self.inner, self.width))
                 self.up_dims = (E, self.inner, self.width)
             if ops.experts_packable(E, self.width, self.inner):
                 self.w_down = ops.pack_matrix(self.w_down.view(E * self.width, self.inner))
                 self.down_dims = (E, self.width, self.inner)
-        self.w_dtype = torch.bfloat16 if isinstance(self.w_gate, ops.PackedMatrix) else self.w_gate.dtype
+        self.w_dtype = torch.bfloat16 if isinstance(self.w_up, ops.PackedMatrix) else self.w_up.dtype
 
     def forward(self, h, ctx, accumulate_into):
         T, top, dev = h.shape[0], self.top, h.device
@@ -188,7 +233,8 @@ class RoutedExperts(Part):
         z = self.router(h, out_dtype=torch.float32)
         ids = torch.empty((T, top), dtype=torch.int32, device=dev)
         wts = torch.empty((T, top), dtype=torch.float32, device=dev)
-        ops.moe_route(z, self.correction, top, ids, wts, score=self.score, renorm=self.renorm, n_experts=self.n_experts)
+        ops.moe_route(z, self.correction, top, ids, wts, score=self.score, renorm=self.renorm, n_experts=self.n_experts,
+                      groups=self.groups, keep=self.keep, scale=self.route_scale)
         offsets = torch.empty(self.n_experts + 1, dtype=torch.int32, device=dev)
         order = torch.empty(T * top, dtype=torch.int32, device=dev)
         ops.moe_plan(ids, self.n_experts, offsets, order)
@@ -202,7 +248,11 @@ class RoutedExperts(Part):
         if self.shared:
             n = self.shared["inner"]
             gu = self.shared_up(h, out_dtype=torch.float32)
-            f = ops.gated(gu[:, n:], gu[:, :n], "silu", torch.empty((T, n), dtype=self.shared_down.weight.dtype, device=dev))
+            f = torch.empty((T, n), dtype=self.shared_down.weight.dtype, device=dev)
+            if self.gated:
+                ops.gated(gu[:, n:], gu[:, :n], "silu", f)
+            else:
+                ops.activate(gu, "relu2", f)
             s = self.shared_down(f, out_dtype=torch.float32)
             if self.token_gate:
                 E = self.n_experts

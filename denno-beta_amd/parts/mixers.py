@@ -28,17 +28,25 @@ class CausalSelfAttention(Part):
     n_heads * value_dim columns.  exact_turn: the projection's result stays 32-bit until queries and keys are turned by
     their positions, so they are rounded once; it is also the way values of another width go (keys and values are then
     kept side by side in one width, the next multiple of 16 from the wider of the two, the narrower padded with zeros,
-    which add nothing to a score or a result)."""
+    which add nothing to a score or a result).  unit_eps: behind the turn every head's q and k are divided by their root
+    mean square, x / sqrt(mean(x^2) + unit_eps) over the head's entries (None: they stay).  head_gate: the name of a matrix
+    [n_heads, width]: head a's result is multiplied by sigmoid(W_g h)_a before the output projection (its rows ride behind
+    the fused projection's; qkv_weight_sources then names the pieces of q, k and v).  Both go the 32-bit way of exact_turn."""
     graph_safe = True
     returns_rows = True
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, scale: float,
                  qkv_weight: str, qkv_bias, out_weight: str, out_bias, stored_in_out: bool = False,
                  window: int = 0, out_init_std: float = 0.02, position=None, qkv_weight_sources=None,
-                 qkv_bias_sources=None, value_dim=None, exact_turn: bool = False):
+                 qkv_bias_sources=None, value_dim=None, exact_turn: bool = False, unit_eps=None, head_gate=None):
         self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim
         self.value_dim = head_dim if value_dim is None else int(value_dim)
-        self.split = bool(exact_turn) or self.value_dim != head_dim
+        self.unit_eps = None if unit_eps is None else float(unit_eps)
+        self.head_gate = head_gate
+        self.split = bool(exact_turn) or self.value_dim != head_dim or self.unit_eps is not None or head_gate is not None
+        if head_gate is not None and (qkv_bias is not None or not qkv_weight_sources or stored_in_out):
+            raise ValueError("causal_attention: a gate per head rides behind a projection without a bias that is stored [out, in] "
+                             "and whose pieces qkv_weight_sources names")
         # (the split way keeps keys and values in one width that every attention kernel takes)
         self.kept_dim = -(-max(head_dim, self.value_dim) // 16) * 16 if self.split else head_dim
         if not 1 <= self.kept_dim <= 256:
@@ -52,7 +60,10 @@ class CausalSelfAttention(Part):
         self.kv_width = n_kv_heads * head_dim
         self.v_width = n_kv_heads * self.value_dim
         # (a checkpoint that stores q, k and v apart names them in qkv_*_sources: joined at load, one product here)
-        self.qkv = Linear(width, self.q_width + self.kv_width + self.v_width, qkv_weight, qkv_bias, stored_in_out,
+        if head_gate is not None:
+            qkv_weight_sources = tuple(qkv_weight_sources) + ((head_gate, n_heads),)
+        self.gate_col = self.q_width + self.kv_width + self.v_width
+        self.qkv = Linear(width, self.gate_col + (n_heads if head_gate is not None else 0), qkv_weight, qkv_bias, stored_in_out,
                           weight_sources=qkv_weight_sources, bias_sources=qkv_bias_sources)
         self.out = Linear(n_heads * self.value_dim, width, out_weight, out_bias, stored_in_out, out_init_std)
         self.position = POSITIONS.make(position) if position is not None else None
@@ -106,14 +117,20 @@ class CausalSelfAttention(Part):
         dims = position.dims if turns else 0
         freq = position.freq if turns else self.no_freq
         # (one launch: queries and keys turned, values moved, each to its place in rows of the kept width)
+        unit = self.unit_eps is not None
         ops.rotary_runs(z, ctx.positions, freq, [(q, 0, H, dk, dims, 0, hw), (kv, self.q_width, G, dk, dims, 0, hw),
-                                                 (kv, self.q_width + self.kv_width, G, dv, 0, G * hw, hw)])
+                                                 (kv, self.q_width + self.kv_width, G, dv, 0, G * hw, hw)],
+                        mag=getattr(position, "mag", 1.0) if turns else 1.0, unit=[unit, unit, False] if unit else None,
+                        eps=self.unit_eps or 0.0)
         if cache.writes:
             ops.kv_write(kv, 0, G * hw, g.slot_map, cache.k, cache.v)
         o = torch.empty((T, H * hw), dtype=act, device=dev)
         ops.attention(q, o, cache.k, cache.v, g.block_tables, g.tiles, H, self.scale, self.window, tiles_wide=g.tiles_wide,
                       single_rows=g.single_rows, max_context=g.max_context)
-        if hw != dv:
+        if self.head_gate is not None:      # (the gate per head, and the heads' first value_dim columns on, in one launch)
+            o = ops.head_gate(o, z[:, self.gate_col:self.gate_col + H], H, dv, torch.empty((T, H * dv), dtype=act, device=dev),
+                              head_stride=hw)
+        elif hw != dv:
             narrow = torch.empty((T, H * dv), dtype=act, device=dev)
             ops.rotary(o, narrow, ctx.positions, self.no_freq, H, 0, dv, src_off=0, src_stride=hw, dst_off=0, dst_stride=dv)
             o = narrow
@@ -170,8 +187,9 @@ class LatentAttention(Part):
     libraries = ("sequence", "grouped")
 
     def __init__(self, width: int, n_heads: int, head_dim: int, rot_dim: int, value_dim: int, kv_rank: int, scale: float,
-                 eps: float, position: dict, names: dict, keep: str = None):
-        """names: q, dkv, g, uk, uv, o (matrices); dkv_norm (vector).
+                 eps: float, position: dict, names: dict, keep: str = None, window: int = 0):
+        """names: q, dkv, g, uk, uv, o (matrices; without "g" the heads' results go on ungated); dkv_norm (vector).
+        window > 0: a query at position p reads the keys p - window + 1 .. p only.
         keep: "latent" (the form above), "heads" (every head's own key [W_uk c | turned part] and value W_uv c are kept,
         as an ordinary attention does: more cache, and the way out where kv_rank + rot_dim is beyond the attention kernels'
         largest head), or None: "latent" where it fits."""
@@ -187,9 +205,15 @@ class LatentAttention(Part):
             raise ValueError(f"latent_attention: a kept key of {kept} numbers; the attention kernels take up to 256")
         self.q_width = n_heads * (head_dim + rot_dim)
         self.o_width = n_heads * value_dim
+        self.window = int(window)
+        self.gated = "g" in names
         # one product for everything that reads h: q | dkv | g
-        self.proj = Linear(width, self.q_width + self.key_dim + self.o_width, names["q"] + "+dkv+g", None,
-                           weight_sources=((names["q"], self.q_width), (names["dkv"], self.key_dim), (names["g"], self.o_width)))
+        if self.gated:
+            self.proj = Linear(width, self.q_width + self.key_dim + self.o_width, names["q"] + "+dkv+g", None,
+                               weight_sources=((names["q"], self.q_width), (names["dkv"], self.key_dim), (names["g"], self.o_width)))
+        else:
+            self.proj = Linear(width, self.q_width + self.key_dim, names["q"] + "+dkv", None,
+                               weight_sources=((names["q"], self.q_width), (names["dkv"], self.key_dim)))
         self.out = Linear(self.o_width, width, names["o"], None)
         self.position = POSITIONS.make(("rotary_pairs", dict(position, head_dim=rot_dim)))
 
@@ -201,7 +225,8 @@ class LatentAttention(Part):
             ParamSpec(self.names["dkv_norm"], (r,), "vector", ("normal", 1.0, 0.1))]
 
     def cache_spec(self):
-        return PagedKV(1, self.key_dim) if self.keep == "latent" else PagedKV(self.n_heads, self.head_width)
+        return (PagedKV(1, self.key_dim, self.window) if self.keep == "latent"
+                else PagedKV(self.n_heads, self.head_width, self.window))
 
     def bind(self, tensors, runtime):
         super().bind(tensors, runtime)
@@ -234,12 +259,18 @@ class LatentAttention(Part):
         ops.heads_linear(z, self.uk_t, q, a_off=0, a_stride=dn + dr, o_off=0, o_stride=kd)
         self.position.turn(z, q, ctx.positions, H, dr, src_off=dn, src_stride=dn + dr, dst_off=r, dst_stride=kd)
         o_lat = torch.empty((T, H * kd), dtype=act, device=h.device)
-        ops.attention(q, o_lat, cache.k, cache.v, g.block_tables, g.tiles, H, self.scale, 0, tiles_wide=g.tiles_wide,
+        ops.attention(q, o_lat, cache.k, cache.v, g.block_tables, g.tiles, H, self.scale, self.window, tiles_wide=g.tiles_wide,
                       single_rows=g.single_rows, max_context=g.max_context)
-        o = torch.empty((T, self.o_width), dtype=torch.float32, device=h.device)
-        ops.heads_linear(o_lat, self.uv, o, a_off=0, a_stride=kd)
-        og = torch.empty((T, self.o_width), dtype=act, device=h.device)
-        ops.gated(o, z[:, gate:], "sigmoid", og)
+        if self.gated:
+            o = torch.empty((T, self.o_width), dtype=torch.float32, device=h.device)
+            ops.heads_linear(o_lat, self.uv, o, a_off=0, a_stride=kd)
+            og = torch.empty((T, self.o_width), dtype=act, device=h.device)
+            ops.gated(o, z[:, gate:], "sigmoid", og)
+        else:
+            og = torch.empty((T, self.o_width), dtype=act, device=h.device)
+            ops.heads_linear(o_lat, self.uv, og, a_off=0, a_stride=kd)
+        if accumulate_into is None:
+            return self.out(og, out_dtype=torch.float32)
         self.out(og, residual=accumulate_into)
 
     def _forward_heads(self, z, ctx, cache, g, accumulate_into):
@@ -261,14 +292,18 @@ class LatentAttention(Part):
         copy(z, q, dn, src_off=0, src_stride=dn + dr, dst_off=0, dst_stride=hw)
         self.position.turn(z, q, ctx.positions, H, dr, src_off=dn, src_stride=dn + dr, dst_off=dn, dst_stride=hw)
         o = torch.empty((T, H * hw), dtype=act, device=dev)
-        ops.attention(q, o, cache.k, cache.v, g.block_tables, g.tiles, H, self.scale, 0, tiles_wide=g.tiles_wide,
+        ops.attention(q, o, cache.k, cache.v, g.block_tables, g.tiles, H, self.scale, self.window, tiles_wide=g.tiles_wide,
                       single_rows=g.single_rows, max_context=g.max_context)
         if hw != dv:
             packed = torch.empty((T, self.o_width), dtype=act, device=dev)
             copy(o, packed, dv, src_off=0, src_stride=hw, dst_off=0, dst_stride=dv)
             o = packed
-        og = torch.empty((T, self.o_width), dtype=act, device=dev)
-        ops.gated(o, z[:, gate:], "sigmoid", og)
+        og = o
+        if self.gated:
+            og = torch.empty((T, self.o_width), dtype=act, device=dev)
+            ops.gated(o, z[:, gate:], "sigmoid", og)
+        if accumulate_into is None:
+            return self.out(og, out_dtype=torch.float32)
         self.out(og, residual=accumulate_into)
 
 

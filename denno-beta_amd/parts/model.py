@@ -74,6 +74,8 @@ class DecoderSpec:
     logit_softcap: float = 0.0            # > 0: then cap * tanh(logit / cap)
     embedding_scale: float = 1.0          # the token table's rows times this, before the position table's
     extra_embeddings: List[EmbeddingTable] = field(default_factory=list)   # added behind them, in this order
+    # further tables that parts of any layer pick rows of: checkpoint name -> (rows, columns); bound into Runtime.tables
+    tables: Dict[str, Tuple[int, int]] = field(default_factory=dict)
     embedding_norm: Optional[PartSpec] = None   # a norm of the embedded rows, before the first layer
     # > 0: the stream is kept as this many copies, all equal to the embedding stage's output at the start and added up
     # behind the last layer; every layer is then of an arrangement that works on copies ("multi_stream")
@@ -205,6 +207,11 @@ class DecoderModel:
             specs.append(ParamSpec(t.name, (t.rows, self.spec.width), "table", ("normal", 0.0, 0.02)))
         for lin in self.injections.values():
             specs += lin.param_specs()
+        for name, (rows, cols) in self.spec.tables.items():
+            if name in seen:
+                raise ValueError(f"two parts claim the tensor {name!r}")
+            seen.add(name)
+            specs.append(ParamSpec(name, (rows, cols), "table", ("normal", 0.0, 1.0)))
         for i, call in enumerate(self.spec.run_order):
             if call.average is not None:
                 specs.append(ParamSpec(call.average, (i + 2,), "vector", ("normal", 1.0 / (i + 2), 0.1)))
@@ -215,6 +222,7 @@ class DecoderModel:
     def bind(self, tensors: Dict[str, torch.Tensor], runtime: Runtime):
         self.runtime = runtime
         runtime.position = self.position          # mixers ask it to turn their queries and keys, if it does that
+        runtime.tables = {name: tensors[name] for name in self.spec.tables}
         for p in self.all_parts():
             p.bind(tensors, runtime)
         self.head.bind(tensors)

@@ -80,7 +80,8 @@ class RMSNorm(Part):
 class StreamRMSNorm(RMSNorm):
     """The norm that stands behind a mixer or a feed-forward, on the result's way into the stream:
     x += mult * (y / sqrt(mean(y^2) + eps) * weight) * scale, with `scale` a vector of the layer's own (a name, or None)
-    and `mult` a constant of the model.  `add_into(y, x)` does it in one kernel; `forward` is the norm alone."""
+    and `mult` a constant of the model.  `add_into(y, x)` does it in one kernel (gate: 32-bit rows z; y is y * sigmoid(z)
+    before the norm, a gate on the sublayer's result); `forward` is the norm alone."""
 
     def __init__(self, width: int, eps: float, weight_name: str, scale_name=None, mult: float = 1.0):
         super().__init__(width, eps, weight_name)
@@ -96,5 +97,5 @@ class StreamRMSNorm(RMSNorm):
         super().bind(tensors, runtime)
         self.scale = tensors[self.scale_name] if self.scale_name else None
 
-    def add_into(self, y, x):
-        return ops.rmsnorm_add(y, self.weight, self.scale, self.mult, self.eps, x)
+    def add_into(self, y, x, gate=None):
+        return ops.rmsnorm_add(y, self.weight, self.scale, self.mult, self.eps, x, gate=gate)

@@ -378,3 +378,77 @@ class Mamba2(Part):
         if accumulate_into is None:
             return self.out(y, out_dtype=F32)
         self.out(y, residual=accumulate_into)
+
+
+@MIXERS.register("mamba1")
+class Mamba1(Part):
+    """The selective scan: a state per channel and state index whose decay the token chooses.  W_in h is laid out
+    [x: inner | z: inner]; x passes a short causal convolution per channel (with a bias) and silu.  W_x x is [dt: dt_rank |
+    B: N | C: N]; the step of a channel is dt_c = log(1 + e^(W_dt dt + bias)_c); A = -e^(A_log), [inner, N].  Per channel c and
+    state index n: S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n; y_c = sum_n S[c, n] C_n + D_c x_c; y times silu(z);
+    then the output projection.  State: S in 32-bit and the convolution's last taps - 1 inputs.  32-bit are the
+    projections' results that enter the recurrence (x behind its convolution, dt, B, C, z), the steps, the decays, the
+    state and its sums; the products' operands are the engine's."""
+    graph_safe = True
+    returns_rows = True
+    libraries = ("sequence",)
+
+    def __init__(self, width: int, inner: int, state_dim: int, dt_rank: int, taps: int, names: dict):
+        """names: in, x, dt, o (matrices); conv [inner, taps], conv_bias, dt_bias, A_log [inner, state_dim], D."""
+        if taps < 1 or inner < 1 or dt_rank < 1 or not 1 <= state_dim <= 256:
+            raise ValueError(f"mamba1: {inner} channels, {state_dim} states (up to 256), a step of rank {dt_rank}, {taps} taps")
+        self.width, self.inner, self.state_dim, self.dt_rank, self.taps, self.names = width, inner, state_dim, dt_rank, taps, dict(names)
+        n = names
+        self.proj = Linear(width, 2 * inner, n["in"], None, init_std=width ** -0.5)
+        self.low = Linear(inner, dt_rank + 2 * state_dim, n["x"], None, init_std=inner ** -0.5)
+        self.step = Linear(dt_rank, inner, n["dt"], n["dt_bias"], init_std=dt_rank ** -0.5)
+        self.out = Linear(inner, width, n["o"], None, init_std=inner ** -0.5)
+
+    def param_specs(self):
+        n = self.names
+        specs = []
+        for lin in (self.proj, self.low, self.step, self.out):
+            specs += lin.param_specs()
+        return specs + [
+            ParamSpec(n["conv"], (self.inner, self.taps), "vector", ("normal", 0.0, 0.4)),
+            ParamSpec(n["conv_bias"], (self.inner,), "vector", ("normal", 0.0, 0.1)),
+            ParamSpec(n["A_log"], (self.inner, self.state_dim), "vector", ("uniform", -2.0, 1.0)),
+            ParamSpec(n["D"], (self.inner,), "vector", ("normal", 1.0, 0.3))]
+
+    def cache_spec(self):
+        return FixedState((self.inner * self.state_dim + (self.taps - 1) * self.inner,))
+
+    def bind(self, tensors, runtime):
+        super().bind(tensors, runtime)
+        for lin in (self.proj, self.low, self.step, self.out):
+            lin.bind(tensors)
+        n = self.names
+        self.conv, self.conv_bias, self.skip = tensors[n["conv"]].contiguous(), tensors[n["conv_bias"]], tensors[n["D"]]
+        self.rates = (-torch.exp(tensors[n["A_log"]].to(F32))).contiguous()       # A, once
+        # the step's product reads the first columns of the rows that W_x left, where those start at 16 bytes
+        per = 16 // (2 if self.step.weight.dtype == torch.bfloat16 else 4)
+        self._view_fits = (self.dt_rank + 2 * self.state_dim) % per == 0
+
+    def forward(self, h, ctx, cache, accumulate_into):
+        act, T, dev = self.runtime.act_dtype, h.shape[0], h.device
+        inner, N, R = self.inner, self.state_dim, self.dt_rank
+        state, past = cache.state[:, :inner * N], cache.state[:, inner * N:]
+        xz = self.proj(h, out_dtype=F32)
+        x = torch.empty((T, inner), dtype=F32, device=dev)
+        ops.conv_rows(xz, self.conv, past, ctx.row_start, ctx.state_slots, x, identity=False, act="silu", bias=self.conv_bias)
+        if self.taps > 1 and cache.writes:
+            ops.history_update(xz[:, :inner], past, ctx.row_start, ctx.state_slots)
+        low = self.low(x, out_dtype=F32)                              # [dt | B | C], 32-bit: B and C enter the recurrence
+        wdt = self.step.weight.dtype
+        dt_in = low[:, :R]
+        if wdt != F32:
+            dt_in = ops.cast(low, torch.empty(low.shape, dtype=wdt, device=dev))[:, :R]
+        if not self._view_fits:
+            dt_in = dt_in.contiguous()
+        dt = self.step(dt_in, out_dtype=F32)                          # (with its bias; the softplus is the scan's)
+        y = torch.empty((T, inner), dtype=act, device=dev)
+        ops.selective_scan(x, dt, None, low[:, R:R + N], low[:, R + N:], self.rates, self.skip, xz[:, inner:], state,
+                           ctx.row_start, ctx.state_slots, y)
+        if accumulate_into is None:
+            return self.out(y, out_dtype=F32)
+        self.out(y, residual=accumulate_into)

@@ -249,6 +249,8 @@ def _act(kind, z, lower=None):
     if kind == "xielu":
         neg = torch.clamp(z, max=0)
         return torch.where(z > 0, lower[0] * z * z + 0.5 * z, lower[1] * (torch.expm1(neg) - neg) + 0.5 * z)
+    if kind == "relu2":
+        return torch.relu(z) ** 2
     raise ValueError(kind)
 
 
@@ -260,8 +262,10 @@ def rmsnorm(x, weight, eps, out, rows=None):
     return out
 
 
-def rmsnorm_add(y, weight, scale, mult, eps, x):
+def rmsnorm_add(y, weight, scale, mult, eps, x, gate=None):
     src = y.float()
+    if gate is not None:
+        src = src * torch.sigmoid(gate.float())
     n = src / torch.sqrt((src * src).mean(dim=-1, keepdim=True) + eps)
     if weight is not None:
         n = n * weight
@@ -325,10 +329,11 @@ def conv_heads(h, w, hist, row_start, slots, out, n_unit, unit_dim, n_first, sca
     return out
 
 
-def rotary_runs(src, positions, freq, runs):
-    for dst, src_off, n_vec, width, dims, dst_off, dst_stride in runs:
+def rotary_runs(src, positions, freq, runs, mag=1.0, unit=None, eps=0.0):
+    unit = [False] * len(runs) if unit is None else unit
+    for (dst, src_off, n_vec, width, dims, dst_off, dst_stride), un in zip(runs, unit):
         rotary(src, dst, positions, freq[:dims // 2], n_vec, dims, width, src_off=src_off, src_stride=width, dst_off=dst_off,
-               dst_stride=dst_stride)
+               dst_stride=dst_stride, mag=mag, unit_eps=eps if un else None)
 
 
 def history_update(h, hist, row_start, slots):
@@ -350,16 +355,19 @@ def shift_mix(h, hist, mu, row_start, slots, out):
     return out
 
 
-def rotary(src, dst, positions, freq, n_vec, dims, width, src_off=0, src_stride=None, dst_off=0, dst_stride=None):
+def rotary(src, dst, positions, freq, n_vec, dims, width, src_off=0, src_stride=None, dst_off=0, dst_stride=None, mag=1.0,
+           unit_eps=None):
     src_stride = width if src_stride is None else src_stride
     dst_stride = width if dst_stride is None else dst_stride
     ang = positions.float()[:, None] * freq[None, :]
-    cos, sin = torch.cos(ang), torch.sin(ang)
+    cos, sin = torch.cos(ang) * mag, torch.sin(ang) * mag
     for n in range(n_vec):
         vec = src[:, src_off + n * src_stride: src_off + n * src_stride + width].float().clone()
         a, b = vec[:, 0:dims:2].clone(), vec[:, 1:dims:2].clone()
         vec[:, 0:dims:2] = a * cos - b * sin
         vec[:, 1:dims:2] = b * cos + a * sin
+        if unit_eps is not None:      # (rotary_runs' norm behind the turn)
+            vec = vec / torch.sqrt((vec * vec).mean(dim=-1, keepdim=True) + unit_eps)
         dst[:, dst_off + n * dst_stride: dst_off + n * dst_stride + width] = vec.to(dst.dtype)
     return dst
 
@@ -446,6 +454,37 @@ def gate_scan(a, b, g, bias_a, bias_b, state, row_start, slots, out):
     return out
 
 
+def head_gate(o, gate, n_heads, dv, out, head_stride=None):
+    hs = dv if head_stride is None else head_stride
+    T = o.shape[0]
+    for h in range(n_heads):
+        out[:, h * dv:(h + 1) * dv] = (o[:, h * hs:h * hs + dv].float() * torch.sigmoid(gate[:, h:h + 1].float())).to(out.dtype)
+    return out
+
+
+def rows_times_table(a, table, ids, off, out):
+    n = a.shape[1]
+    out.copy_(a.float() * table[ids.long(), off:off + n].float())
+    return out
+
+
+def selective_scan(x, dt, dt_bias, B, C, A, D, z, state, row_start, slots, out):
+    inner, N = A.shape
+    step = torch.nn.functional.softplus(dt.double() + (dt_bias.double() if dt_bias is not None else 0.0))
+    for slot, lo, hi in _requests(row_start, slots):
+        S = state[slot].double().view(inner, N).clone()
+        for t in range(lo, hi):
+            S = torch.exp(step[t][:, None] * A.double()) * S + (step[t] * x[t].double())[:, None] * B[t].double()[None, :]
+            y = S @ C[t].double()
+            if D is not None:
+                y = y + D.double() * x[t].double()
+            if z is not None:
+                y = y * _act("silu", z[t].double())
+            out[t] = y.to(out.dtype)
+        state[slot] = S.reshape(-1).to(state.dtype)
+    return out
+
+
 def streams_read(xs, w_in, weight, eps, out, rows=None):
     n = xs.shape[0]
     u = sum((w_in[s].double() if w_in is not None else 1.0) * xs[s].double() for s in range(n))
@@ -511,13 +550,22 @@ def heads_linear(a, w, out, a_off=0, a_stride=None, o_off=0, o_stride=None):
     return out
 
 
-def moe_route(z, correction, top, ids, wts, score="softmax", renorm=True, n_experts=None):
+def moe_route(z, correction, top, ids, wts, score="softmax", renorm=True, n_experts=None, groups=1, keep=1, scale=1.0):
     if n_experts is not None:
         z = z[:, :n_experts]
+    E = z.shape[1]
     s = torch.softmax(z, dim=-1) if score == "softmax" else torch.sigmoid(z)
     choice = s if correction is None else s + correction
     for t in range(z.shape[0]):
         c = choice[t].clone()
+        if keep < groups:
+            per = E // groups
+            gs = c.view(groups, per).topk(min(2, per), dim=-1).values.sum(dim=-1)
+            closed = torch.ones(groups, dtype=torch.bool)
+            for _ in range(keep):
+                g = int(torch.argmax(torch.where(closed, gs, torch.full_like(gs, -float("inf")))))
+                closed[g] = False
+            c[closed.repeat_interleave(per)] = -float("inf")
         picked = []
         for _ in range(top):
             e = int(torch.argmax(c))           # (the first of equal values)
@@ -525,7 +573,7 @@ def moe_route(z, correction, top, ids, wts, score="softmax", renorm=True, n_expe
             c[e] = -float("inf")
         ws = s[t, picked]
         ids[t] = torch.tensor(picked, dtype=torch.int32)
-        wts[t] = ws / (ws.sum() + 1e-20) if renorm else ws
+        wts[t] = (ws / (ws.sum() + 1e-20) if renorm else ws) * scale
 
 
 def moe_plan(ids, n_experts, offsets, order):
@@ -540,9 +588,13 @@ def moe_plan(ids, n_experts, offsets, order):
 def moe_up(h, order, offsets, top, w_gate, w_up, limit, alpha, y, dims=None, kind="clamped", in_scale=None):
     assert dims is None, "packed experts are for the GPU's kernels"
     off = offsets.tolist()
-    for e in range(w_gate.shape[0]):
+    for e in range(w_up.shape[0]):
         for p in range(off[e], off[e + 1]):
             x = h[int(order[p]) // top].float()
+            if kind == "relu2":
+                sc = 1.0 if in_scale is None else in_scale.reshape(-1)[int(order[p])]
+                y[p] = (torch.relu((w_up[e].float() @ x) * sc) ** 2).to(y.dtype)
+                continue
             if kind == "silu":
                 sc = 1.0 if in_scale is None else in_scale.reshape(-1)[int(order[p])]
                 g, u = (w_gate[e].float() @ x) * sc, (w_up[e].float() @ x) * sc
