@@ -548,3 +548,146 @@ def test_queries_and_keys_normed_whole_and_written_to_the_cache(dtype, H, Hkv, d
     args = make() + (False,)
     ops.norm_pair_write(*args)
     assert float(args[7].float().abs().sum()) == 0.0 and float(args[8].float().abs().sum()) == 0.0
+
+
+# ---- a state per channel and state index, gates on results, rows of a table, routing in groups, experts without a gate ----
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("inner,N,lengths", [(16, 16, [5]), (37, 1, [1, 9, 1]), (50, 5, [3, 1, 40]), (24, 24, [1, 1, 1, 1]), (19, 40, [33, 2]),
+                                             (8, 100, [7, 12]), (5, 256, [6]), (130, 8, [70])])
+def test_selective_scan(dtype, inner, N, lengths):
+    row_start, slots, T = tables(lengths, ([3, -1, 0, 2, 1] * 2)[:len(lengths)] if len(lengths) > 1 else [1])
+    wide = torch.randn(T, 2 * inner + 3, device=DEV)                       # x and z as columns of wider rows
+    low = torch.randn(T, 4 + 2 * N, device=DEV)
+    dt = torch.randn(T, inner, device=DEV) * 2 - 1
+    A = -torch.exp(torch.rand(inner, N, device=DEV) * 4 - 3)
+    D, bias = torch.randn(inner, device=DEV), torch.randn(inner, device=DEV)
+
+    def make(z, d, b):
+        state = torch.randn(5, inner * N + 7, device=DEV)[:, :inner * N]
+        return (wide[:, :inner], dt, b, low[:, 4:4 + N], low[:, 4 + N:], A, d, z, state, row_start, slots,
+                torch.zeros(T, inner, dtype=dtype, device=DEV))
+    keep = torch.random.get_rng_state(), torch.cuda.get_rng_state()
+    for z, d, b in ((wide[:, inner + 3:], D, bias), (None, None, None)):
+        torch.random.set_rng_state(keep[0]), torch.cuda.set_rng_state(keep[1])
+        args = make(z, d, b)
+        host = [a.detach().cpu().clone() if isinstance(a, torch.Tensor) else a for a in args]
+        ops.selective_scan(*args)
+        ref.selective_scan(*host)
+        live = [i for i, s in enumerate(slots.tolist()) if s >= 0]
+        rows = torch.cat([torch.arange(row_start[i], row_start[i + 1]) for i in live])
+        close(args[11][rows], host[11][rows], dtype, "selective_scan rows")
+        close(args[8], host[8], torch.float32, "selective_scan state")
+        assert float(args[11][[r for r in range(T) if r not in rows.tolist()]].abs().sum()) == 0.0      # (padding is left alone)
+
+
+def test_selective_scan_cut_anywhere_gives_the_same_bits():
+    inner, N, T = 21, 12, 47
+    x, dt, z = (torch.randn(T, inner, device=DEV) for _ in range(3))
+    B, C = torch.randn(T, N, device=DEV), torch.randn(T, N, device=DEV)
+    A = -torch.exp(torch.rand(inner, N, device=DEV) * 3 - 2)
+    D = torch.randn(inner, device=DEV)
+    one = torch.tensor([0], dtype=torch.int32, device=DEV)
+
+    def run(cuts):
+        state, out = torch.zeros(1, inner * N, device=DEV), torch.zeros(T, inner, device=DEV)
+        for a, b in zip(cuts[:-1], cuts[1:]):
+            rs = torch.tensor([0, b - a], dtype=torch.int32, device=DEV)
+            ops.selective_scan(x[a:b], dt[a:b], None, B[a:b], C[a:b], A, D, z[a:b], state, rs, one, out[a:b])
+        return out, state
+    whole = run([0, T])
+    for cuts in ([0, 1, 2, 3, T], [0, 5, 7, 40, 41, T], list(range(T + 1))):
+        got = run(cuts)
+        assert torch.equal(got[0], whole[0]) and torch.equal(got[1], whole[1]), cuts
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("width", [9, 64, 700])
+def test_norm_of_a_gated_result_added_into_the_stream(width, dtype):
+    T = 11
+    y = (torch.randn(T, width, device=DEV) * 2).to(dtype)
+    gate = torch.randn(T, width + 3, device=DEV)[:, :width] * 2
+    w = torch.randn(width, device=DEV)
+    x = torch.randn(T, width, device=DEV)
+    hx = x.cpu().clone()
+    ops.rmsnorm_add(y, w, None, 1.0, 1e-5, x, gate=gate)
+    ref.rmsnorm_add(y.cpu(), w.cpu(), None, 1.0, 1e-5, hx, gate=gate.cpu())
+    close(x, hx)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("H,G,dk,dv,dims,hw", [(4, 2, 16, 8, 8, 16), (3, 1, 24, 40, 24, 48), (2, 2, 10, 6, 4, 16), (5, 5, 256, 32, 64, 256),
+                                               (1, 1, 3, 2, 2, 16)])
+def test_runs_turned_and_normed_in_one_launch(dtype, H, G, dk, dv, dims, hw):
+    T = 9
+    z = torch.randn(T, H * dk + G * dk + G * dv + 2, device=DEV) * 2
+    pos = torch.randint(0, 5000, (T,), dtype=torch.int32, device=DEV)
+    freq = (10000.0 ** (-torch.arange(dims // 2, dtype=torch.float64) * 2 / dims)).float().to(DEV)
+    for mag, unit in ((1.0, [True, True, False]), (1.07, [True, False, False]), (0.9, None)):
+        q, kv = torch.zeros(T, H * hw, dtype=dtype, device=DEV), torch.zeros(T, 2 * G * hw, dtype=dtype, device=DEV)
+        hq, hkv = q.cpu().clone(), kv.cpu().clone()
+        runs = lambda a, b: [(a, 0, H, dk, dims, 0, hw), (b, H * dk, G, dk, dims, 0, hw), (b, H * dk + G * dk, G, dv, 0, G * hw, hw)]  # noqa: E731
+        ops.rotary_runs(z, pos, freq, runs(q, kv), mag=mag, unit=unit, eps=1e-5)
+        ref.rotary_runs(z.cpu(), pos.cpu(), freq.cpu(), runs(hq, hkv), mag=mag, unit=unit, eps=1e-5)
+        close(q, hq, dtype, "queries"), close(kv, hkv, dtype, "keys and values")
+    if dk <= 64:
+        # a normed vector has a root mean square of one whatever its position
+        qf = torch.zeros(T, H * hw, device=DEV)
+        ops.rotary_runs(z, pos, freq, [(qf, 0, H, dk, dims, 0, hw)], mag=1.3, unit=[True], eps=0.0)
+        rms = qf.view(T, H, hw)[:, :, :dk].pow(2).mean(-1).sqrt()
+        assert float((rms - 1).abs().max()) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", DT)
+def test_a_gate_per_head_and_rows_times_a_table(dtype):
+    T, H, dv, hs = 7, 3, 10, 16
+    o = torch.randn(T, H * hs, device=DEV).to(dtype)
+    g = torch.randn(T, H + 5, device=DEV)[:, 2:2 + H]
+    both("head_gate", lambda: (o, g, H, dv, torch.zeros(T, H * dv, dtype=dtype, device=DEV), hs), [4], dtype)
+    both("head_gate", lambda: (o[:, :H * dv], g, H, dv, torch.zeros(T, H * dv, dtype=dtype, device=DEV)), [4], dtype)
+    table = torch.randn(23, 40, device=DEV).to(dtype)
+    a = torch.randn(T, 12, device=DEV).to(dtype)
+    ids = torch.randint(0, 23, (T,), dtype=torch.int32, device=DEV)
+    both("rows_times_table", lambda: (a, table, ids, 17, torch.zeros(T, 12, dtype=dtype, device=DEV)), [4], dtype)
+    want = a.float() * table.float()[ids.long(), 28:40]
+    got = ops.rows_times_table(a, table, ids, 28, torch.zeros(T, 12, dtype=dtype, device=DEV))
+    close(got, want, dtype)
+
+
+@pytest.mark.parametrize("T,E,top,groups,keep", [(40, 8, 3, 2, 1), (17, 12, 2, 3, 2), (9, 6, 1, 6, 2), (33, 64, 4, 8, 3), (5, 192, 6, 4, 1),
+                                                 (12, 10, 10, 5, 5), (7, 9, 2, 1, 1)])
+def test_route_inside_the_best_groups(T, E, top, groups, keep):
+    z = torch.randn(T, E, device=DEV) * 2
+    corr = torch.randn(E, device=DEV) * 0.1
+    for score, renorm, scale, c in (("sigmoid", True, 2.5, None), ("softmax", False, 1.0, corr), ("sigmoid", True, 1.0, corr)):
+        ids, wts = torch.zeros(T, top, dtype=torch.int32, device=DEV), torch.zeros(T, top, device=DEV)
+        ops.moe_route(z, c, top, ids, wts, score=score, renorm=renorm, groups=groups, keep=keep, scale=scale)
+        hi, hw = torch.zeros(T, top, dtype=torch.int32), torch.zeros(T, top)
+        ref.moe_route(z.cpu(), None if c is None else c.cpu(), top, hi, hw, score=score, renorm=renorm, groups=groups, keep=keep, scale=scale)
+        assert torch.equal(ids.cpu(), hi), (score, ids.cpu()[:3], hi[:3])
+        close(wts, hw)
+        # every choice lies in one of at most `keep` groups
+        assert int((ids.cpu() // (E // groups)).sort(dim=1).values.diff(dim=1).ne(0).sum(dim=1).max()) + 1 <= keep if top > 1 else True
+        if renorm:
+            close(wts.sum(dim=1), torch.full((T,), scale))
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("T,E,top,ff,width", [(1, 3, 2, 8, 24), (45, 6, 3, 70, 50), (200, 5, 2, 64, 128), (9, 8, 2, 96, 64), (3, 40, 1, 32, 160)])
+def test_experts_without_a_gate(dtype, T, E, top, ff, width):
+    """max(W_up h, 0)^2 through the plain kernel, the matrix-core kernel and the one for packed weights."""
+    h = torch.randn(T, width, device=DEV).to(dtype)
+    wu = (torch.randn(E, ff, width, device=DEV) / width ** 0.5).to(dtype)
+    ids = torch.stack([torch.randperm(E, device=DEV)[:top] for _ in range(T)]).int()
+    offsets, order = torch.zeros(E + 1, dtype=torch.int32, device=DEV), torch.zeros(T * top, dtype=torch.int32, device=DEV)
+    ops.moe_plan(ids, E, offsets, order)
+    y = torch.zeros(T * top, ff, dtype=dtype, device=DEV)
+    ops.moe_up(h, order, offsets, top, None, wu, 0.0, 1.0, y, kind="relu2")
+    hy = torch.zeros(T * top, ff, dtype=dtype)
+    ref.moe_up(h.cpu(), order.cpu(), offsets.cpu(), top, None, wu.cpu(), 0.0, 1.0, hy, kind="relu2")
+    close(y, hy, dtype, "moe_up")
+    if dtype == torch.bfloat16 and ops.experts_packable(E, ff, width):
+        y2 = torch.zeros_like(y)
+        ops.moe_up(h, order, offsets, top, None, ops.pack_matrix(wu.view(E * ff, width)), 0.0, 1.0, y2, dims=(E, ff, width), kind="relu2")
+        close(y2, hy, dtype, "moe_up, packed")
+    z = torch.randn(T, ff, device=DEV)
+    close(ops.activate(z, "relu2", torch.zeros(T, ff, dtype=dtype, device=DEV)), torch.relu(z) ** 2, dtype)
