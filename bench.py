@@ -25,6 +25,11 @@ decode steps and prefill (`fp32`).  Peaks are the published ones of MI355X.
                                                              Mamba2, Mamba2, the pair again; dense feed-forwards; the stream in two
                                                              copies) beside four Pafivik layers with dense feed-forwards of the same
                                                              width (attention, lightning, lightning, attention): prefill and decode
+    python bench.py --only nigilorn [--width 1024] [--kernel-times]  four Nigilorn layers (selective scan, attention in a window,
+                                                             latent attention in a window, selective scan; a dense feed-forward, then
+                                                             sixteen experts and a shared one; gated sublayers, a token input behind
+                                                             every layer) beside four Pafivik layers of the same width and feed-forward
+                                                             sizes (lightning, attention, attention, lightning): prefill and decode
 """
 import argparse
 import json
@@ -194,8 +199,8 @@ def main():
     ap.add_argument("--shape", choices=["xl", "large", "medium"], default=None,
                     help="--only decode / prefill / replay: the layer sizes of BASELINE.json's configs[2], [3] or [4] "
                          "(default xl; for replay medium)")
-    ap.add_argument("--width", type=int, default=0, help="--only ridopel, pafivik, dogalorn: one width instead of 1,024 and 2,048")
-    ap.add_argument("--only", choices=["decode", "prefill", "serving", "replay", "ridopel", "pafivik", "dogalorn"], default=None,
+    ap.add_argument("--width", type=int, default=0, help="--only ridopel, pafivik, dogalorn, nigilorn: one width instead of 1,024 and 2,048")
+    ap.add_argument("--only", choices=["decode", "prefill", "serving", "replay", "ridopel", "pafivik", "dogalorn", "nigilorn"], default=None,
                     help="run one workload and print a short line (decode, prefill: for profiling; serving: "
                          "BASELINE.json's configs[3], GPT-2 Large shape, 64 requests through the scheduler; replay: "
                          "configs[4], GPT-2 Medium shape, against the plain implementation)")
@@ -211,6 +216,8 @@ def main():
         return pafivik(a)
     if a.only == "dogalorn":
         return dogalorn(a)
+    if a.only == "nigilorn":
+        return nigilorn(a)
     if a.only == "replay":
         a.shape = a.shape or "medium"      # (configs[4] as written; --shape xl: the same replay at configs[2]'s sizes)
         return replay(a)
@@ -333,6 +340,43 @@ def dogalorn_configs(width, layers=4, vocab=32000, positions=2048):
     paf = dict(architecture="Pafivik", vocab=vocab, width=width, norm=dict(eps=1e-5), embedding=dict(scale=1.0), residual_mult=0.5,
                layers=[kinds[i % 4] for i in range(layers)], max_positions=positions, n_positions=positions, vocab_size=vocab)
     return dog, paf
+
+
+def nigilorn_configs(width, layers=4, vocab=32000, positions=2048):
+    """-> (a Nigilorn config, a Pafivik config) of the same width, layers, vocabulary and positions.  The Nigilorn layers: a
+    selective scan (twice the width in channels, 16 states a channel, a step of rank width / 16, four taps); attention
+    (heads of 64, a key head for every four, half of a head turned with a stretched encoding, a window of 256); latent
+    attention (heads of 64 + 32, values of 128, a kept key of 224 + 32 numbers, a window of 256); the scan again.  The first
+    layer has a dense feed-forward of four times the width, the others sixteen experts of the model's width in four groups
+    of which two are kept, two experts a token, and a shared expert of the model's width; a token input of 64 columns a
+    layer.  The Pafivik layers (lightning, attention, attention, lightning) have the same feed-forward sizes."""
+    H = width // 64
+    stretch = dict(factor=4.0, original=512, fast=32.0, slow=1.0)
+    ff = dict(kind="dense", ff=4 * width)
+    moe = dict(kind="moe", expert=dict(ff=width), router=dict(experts=16, top=2, scale=2.5, groups=dict(count=4, keep=2)), shared=dict(ff=width))
+    scan = dict(type="mamba1", mixer=dict(inner=2 * width, state=16, dt_rank=width // 16, conv=4))
+    att = dict(type="attention", mixer=dict(heads=H, kv_heads=max(1, H // 4), dim=64, vdim=64, scale=0.125, mask=dict(size=256),
+                                            rot=dict(base=10000.0, dims=32, scaling=stretch)))
+    lat = dict(type="latent_attention", mixer=dict(heads=width // 128, dim=64, rot_dim=32, vdim=128, kv_rank=224, scale=96 ** -0.5,
+                                                   mask=dict(size=256), rot=dict(base=10000.0, dims=32, scaling=stretch)))
+    kinds = [dict(scan, mlp=ff), dict(att, mlp=moe), dict(lat, mlp=moe), dict(scan, mlp=moe)]
+    nig = dict(architecture="Nigilorn", vocab=vocab, width=width, norm=dict(eps=1e-5), token_side=dict(dim=64),
+               layers=[kinds[i % 4] for i in range(layers)], max_positions=positions, n_positions=positions, vocab_size=vocab)
+    Hl = width // 128
+    pmoe = dict(kind="moe", expert=dict(ff=width), router=dict(experts=16, top=2), shared=dict(ff=width))
+    patt = dict(type="attention", mixer=dict(heads=H, kv_heads=max(1, H // 4), dim=64, vdim=64, scale=0.125, rot=dict(base=10000.0, dims=64)))
+    lig = dict(type="lightning", mixer=dict(heads=Hl, dim=64, vdim=128, decay=[1.0 - 2.0 ** -(5 + 3 * h / Hl) for h in range(Hl)]))
+    kinds = [dict(lig, mlp=ff), dict(patt, mlp=pmoe), dict(patt, mlp=pmoe), dict(lig, mlp=pmoe)]
+    paf = dict(architecture="Pafivik", vocab=vocab, width=width, norm=dict(eps=1e-5), embedding=dict(scale=1.0), residual_mult=0.5,
+               layers=[kinds[i % 4] for i in range(layers)], max_positions=positions, n_positions=positions, vocab_size=vocab)
+    return nig, paf
+
+
+def nigilorn(a):
+    """Prefill and decode steps of four Nigilorn layers beside four Pafivik layers of the same width and feed-forward sizes
+    (the closest of the framework's models: a norm on both sides of every sublayer, an attention over pages, a recurrence
+    with a state, experts with a shared one); with --kernel-times each model's kernels."""
+    return side_by_side(a, ("nigilorn", "pafivik"), nigilorn_configs)
 
 
 def dogalorn(a):
