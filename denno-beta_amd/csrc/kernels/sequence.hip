@@ -888,6 +888,144 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(SelectiveArgs a) {
   }
 }
 
+// lane i's value of each row of 16 lanes, in all lanes of the row (i is a constant once the caller's loop is unrolled)
+__device__ __forceinline__ float row_share(float v, int i) {
+  switch (i & 15) {
+    case 0: return dpp_move<0x150>(v);
+    case 1: return dpp_move<0x151>(v);
+    case 2: return dpp_move<0x152>(v);
+    case 3: return dpp_move<0x153>(v);
+    case 4: return dpp_move<0x154>(v);
+    case 5: return dpp_move<0x155>(v);
+    case 6: return dpp_move<0x156>(v);
+    case 7: return dpp_move<0x157>(v);
+    case 8: return dpp_move<0x158>(v);
+    case 9: return dpp_move<0x159>(v);
+    case 10: return dpp_move<0x15A>(v);
+    case 11: return dpp_move<0x15B>(v);
+    case 12: return dpp_move<0x15C>(v);
+    case 13: return dpp_move<0x15D>(v);
+    case 14: return dpp_move<0x15E>(v);
+    default: return dpp_move<0x15F>(v);
+  }
+}
+
+// The same recurrence for long portions of few requests, where a wave that walks a request's rows alone leaves the chip
+// idle: a workgroup's WAVES waves take TB rows each (TB <= 8) of every run of WAVES * TB rows.  A wave first walks its
+// rows from a state of zero, which gives, per state, the product P of its decays and what it adds, Q, so that the state
+// behind its rows is P S + Q for any state S before them; the waves' (P, Q) meet in LDS, every wave folds those of the
+// waves before it into the state at the run's start, in order, and walks its rows again from there (the decays and
+// summands are kept from the first walk).  What is one number per row and channel is made once, not by all 16 lanes of
+// the channel: lane i of them (i < TB) has row i's step (softplus) and step * x, lane 8 + i its silu(z) and x, and the
+// others read them from there (DPP row_share).  The decays are 2^(step * A log2(e)) by the hardware's exponential.
+// A row's result depends on the rows before it alone; how the rows were cut changes it by rounding only, where the
+// kernel above gives the same bits.
+template <int PER, int WAVES, int TB>
+__global__ __launch_bounds__(WAVES * 64) void selective_scan_runs_kernel(SelectiveArgs a) {
+  static_assert(TB <= 8, "a row's step lies on lane i, its gate on lane 8 + i of the channel's 16");
+  __shared__ float shp[2][WAVES][PER][64], shq[2][WAVES][PER][64];
+  const int s = blockIdx.y;
+  const int slot = a.slots[s];
+  if (slot < 0) return;      // (the whole workgroup)
+  const int row0 = a.row_start[s], row1 = a.row_start[s + 1];
+  if (row0 >= row1) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l = lane & 15;
+  const int c = blockIdx.x * 4 + (lane >> 4);
+  const bool live = c < a.inner;
+  const int cc = live ? c : a.inner - 1;
+  float rate[PER], S0[PER];
+  int nn[PER];
+  float* sp = a.state + static_cast<size_t>(slot) * a.slot_stride + static_cast<size_t>(cc) * a.N;
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int n = l + 16 * j;
+    const bool has = n < a.N;
+    nn[j] = has ? n : 0;
+    rate[j] = has ? a.A[static_cast<size_t>(cc) * a.N + n] * 1.4426950408889634f : 0.f;
+    S0[j] = has ? sp[n] : 0.f;      // the state before the run that is worked on; every wave keeps it
+  }
+  const float bias = a.dt_bias ? a.dt_bias[cc] : 0.f, skip = a.D ? a.D[cc] : 0.f;
+  const bool steps = l < 8;              // this lane makes a row's step; else its gate
+  const int my = l & 7;                  // the row of the wave's TB that this lane makes them for
+  float fx, fs, fb[TB][PER], fc[TB][PER];
+  auto fetch = [&](int t0) {
+    const size_t t = min(t0 + min(my, TB - 1), row1 - 1);
+    fx = a.x[t * a.ldx + cc];
+    fs = steps ? a.dt[t * a.ldd + cc] : (a.z ? a.z[t * a.ldz + cc] : 0.f);
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      const size_t r = min(t0 + i, row1 - 1);
+#pragma unroll
+      for (int j = 0; j < PER; ++j) fb[i][j] = a.B[r * a.ldb + nn[j]], fc[i][j] = a.C[r * a.ldc + nn[j]];
+    }
+  };
+  fetch(row0 + wave * TB);
+  int par = 0;
+  for (int t0 = row0; t0 < row1; t0 += WAVES * TB, par ^= 1) {
+    const int mine = t0 + wave * TB;
+    // lanes 0 .. 7: (step, step * x) of row `my`; lanes 8 .. 15: (silu(z) or 1, D x) of row `my`
+    float first, second;
+    if (steps) {
+      first = softplus_f(fs + bias);
+      second = first * fx;
+    } else {
+      first = a.z ? fs / (1.0f + expf(-fs)) : 1.0f;
+      second = skip * fx;
+    }
+    float keep[TB][PER], add[TB][PER], cm[TB][PER];
+    float P[PER], Q[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) P[j] = 1.f, Q[j] = 0.f;
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      const bool row = mine + i < row1;
+      const float dt = row_share(first, i), dx = row_share(second, i);
+#pragma unroll
+      for (int j = 0; j < PER; ++j) {
+        const bool has = l + 16 * j < a.N;
+        keep[i][j] = row ? __builtin_amdgcn_exp2f(dt * rate[j]) : 1.0f;      // (places beyond the last row change nothing)
+        add[i][j] = (row && has) ? dx * fb[i][j] : 0.f;
+        cm[i][j] = has ? fc[i][j] : 0.f;
+        P[j] *= keep[i][j];
+        Q[j] = fmaf(keep[i][j], Q[j], add[i][j]);
+      }
+    }
+    if (t0 + WAVES * TB < row1) fetch(mine + WAVES * TB);
+    float S[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) shp[par][wave][j][lane] = P[j], shq[par][wave][j][lane] = Q[j];
+    __syncthreads();      // (the other half of LDS is what the run before used: one barrier a run)
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      float run = S0[j];
+      S[j] = run;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) {
+        if (w == wave) S[j] = run;
+        run = fmaf(shp[par][w][j][lane], run, shq[par][w][j][lane]);
+      }
+      S0[j] = run;
+    }
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      float y = 0.f;
+#pragma unroll
+      for (int j = 0; j < PER; ++j) {
+        S[j] = fmaf(keep[i][j], S[j], add[i][j]);
+        y = fmaf(S[j], cm[i][j], y);
+      }
+      y = group_reduce<16>(y, SumOp());
+      const float gate = row_share(first, 8 + i), dx = row_share(second, 8 + i);
+      if (live && l == 0 && mine + i < row1) store_as(a.out, static_cast<size_t>(mine + i) * a.ldo + c, a.out_dt, (y + dx) * gate);
+    }
+  }
+  if (live && wave == 0) {
+#pragma unroll
+    for (int j = 0; j < PER; ++j)
+      if (l + 16 * j < a.N) sp[l + 16 * j] = S0[j];
+  }
+}
+
 // ---- queries and keys normed as whole vectors, keys and values to the cache -----------------------------------------
 // A row of z is [q: qw | k: kw].  q_out[t] = q / rms(q) * wq; the key that goes to the cache is k / rms(k) * wk, the value
 // k as it is (pools [page][key head][offset][dim] and [page][key head][dim][offset], the row's place from slot_map; a
@@ -1416,16 +1554,24 @@ int dn_rows_times_table(const void* a, int a_dt, long long lda, const void* tabl
 
 int dn_selective_scan(const float* x, long long ldx, const float* dt, long long ldd, const float* dt_bias, const float* B, long long ldb,
                       const float* C, long long ldc, const float* A, const float* D, const float* z, long long ldz, float* state,
-                      long long slot_stride, const int* row_start, const int* slots, int S, int inner, int N, void* out, int out_dt,
-                      long long ldo, hipStream_t stream) {
+                      long long slot_stride, const int* row_start, const int* slots, int S, int T, int inner, int N, void* out,
+                      int out_dt, long long ldo, int in_order, hipStream_t stream) {
   if (!float_kind(out_dt)) return DN_ERR_DTYPE;
   if (inner < 1 || N < 1 || N > 256 || S > 65535 || slot_stride < static_cast<long long>(inner) * N) return DN_ERR_SHAPE;
   if (S == 0) return 0;
   const SelectiveArgs a{x, dt, dt_bias, B, C, A, D, z, static_cast<size_t>(ldx), static_cast<size_t>(ldd), static_cast<size_t>(ldb),
                         static_cast<size_t>(ldc), static_cast<size_t>(ldz), state, static_cast<size_t>(slot_stride), row_start, slots,
                         inner, N, out, out_dt, static_cast<size_t>(ldo)};
-  const dim3 grid((inner + 15) / 16, S);
   const int per = (N + 15) / 16;
+  // (portions of few requests: the rows shared out among eight waves, which leaves a wave the registers of half a SIMD; up to four states a lane)
+  if (!in_order && per <= 4 && T > 32 * S && static_cast<long long>(S) * ((inner + 15) / 16) < 2048) {
+    const dim3 runs((inner + 3) / 4, S);
+    if (per <= 1) hipLaunchKernelGGL((selective_scan_runs_kernel<1, 8, 8>), runs, dim3(512), 0, stream, a);
+    else if (per <= 2) hipLaunchKernelGGL((selective_scan_runs_kernel<2, 8, 4>), runs, dim3(512), 0, stream, a);
+    else hipLaunchKernelGGL((selective_scan_runs_kernel<4, 8, 2>), runs, dim3(512), 0, stream, a);
+    return dn_launch_status();
+  }
+  const dim3 grid((inner + 15) / 16, S);
   if (per <= 1) hipLaunchKernelGGL(selective_scan_kernel<1>, grid, dim3(256), 0, stream, a);
   else if (per <= 2) hipLaunchKernelGGL(selective_scan_kernel<2>, grid, dim3(256), 0, stream, a);
   else if (per <= 4) hipLaunchKernelGGL(selective_scan_kernel<4>, grid, dim3(256), 0, stream, a);

@@ -152,7 +152,7 @@ def _declare(name, lib):
             "dn_head_gate": [P, I, c_longlong, I, P, c_longlong, P, I, c_longlong, I, I, I, P],
             "dn_rows_times_table": [P, I, c_longlong, P, I, c_longlong, I, P, I, P, I, c_longlong, I, I, P],
             "dn_selective_scan": [P, c_longlong, P, c_longlong, P, P, c_longlong, P, c_longlong, P, P, P, c_longlong, P, c_longlong,
-                                  P, P, I, I, I, P, I, c_longlong, P],
+                                  P, P, I, I, I, I, P, I, c_longlong, I, P],
         },
         "grouped": {
             "dn_heads_linear": [P, I, c_longlong, I, I, P, I, P, I, c_longlong, I, I, I, I, I, I, P],
@@ -1321,12 +1321,14 @@ def rows_times_table(a, table, ids, off, out):
     return out
 
 
-def selective_scan(x, dt, dt_bias, B, C, A, D, z, state, row_start, slots, out):
+def selective_scan(x, dt, dt_bias, B, C, A, D, z, state, row_start, slots, out, in_order=False):
     """A state per channel c and state index n with a decay of its own, over each request's rows in order:
       step = log(1 + e^(dt[t, c] + dt_bias[c]));  S[c, n] <- exp(step * A[c, n]) S[c, n] + step * x[t, c] * B[t, n]
       y[t, c] = sum_n S[c, n] C[t, n] + D[c] x[t, c];  out[t, c] = y * silu(z[t, c])      (z None: y as it is)
     x, dt, z: 32-bit [T, inner]; B, C: 32-bit [T, N] (all may be columns of wider rows); A: 32-bit [inner, N]; dt_bias, D:
-    32-bit [inner] or None; state: 32-bit [slots, inner * N], read and written at the requests' slots; out [T, inner]."""
+    32-bit [inner] or None; state: 32-bit [slots, inner * N], read and written at the requests' slots; out [T, inner].
+    in_order: every request's rows are walked one after the other, which gives the same bits however a prompt is cut; else
+    long portions of few requests are shared out among a workgroup's waves and joined, which changes a result by rounding."""
     for t, name in ((x, "x"), (dt, "dt"), (B, "B"), (C, "C")) + (((z, "z"),) if z is not None else ()):
         _dev(t, name, (torch.float32,), 2)
     _dev(out, "out", _FLOATS, 2), _dev(A, "A", (torch.float32,), 2)
@@ -1341,8 +1343,8 @@ def selective_scan(x, dt, dt_bias, B, C, A, D, z, state, row_start, slots, out):
     _ok(_lib("sequence").dn_selective_scan(x.data_ptr(), _rows(x, "x"), dt.data_ptr(), _rows(dt, "dt"), _ptr(dt_bias), B.data_ptr(),
                                            _rows(B, "B"), C.data_ptr(), _rows(C, "C"), A.data_ptr(), _ptr(D), _ptr(z),
                                            _rows(z, "z") if z is not None else 0, state.data_ptr(), stride, row_start.data_ptr(),
-                                           slots.data_ptr(), S, inner, N, out.data_ptr(), _CODE[out.dtype], _rows(out, "out"),
-                                           _stream()), "selective_scan")
+                                           slots.data_ptr(), S, T, inner, N, out.data_ptr(), _CODE[out.dtype], _rows(out, "out"),
+                                           int(bool(in_order)), _stream()), "selective_scan")
     return out
 
 

@@ -447,8 +447,9 @@ class Mamba1(Part):
             dt_in = dt_in.contiguous()
         dt = self.step(dt_in, out_dtype=F32)                          # (with its bias; the softplus is the scan's)
         y = torch.empty((T, inner), dtype=act, device=dev)
+        # (the 32-bit engine walks a request's rows in order: its logits are the same bits however a prompt is cut)
         ops.selective_scan(x, dt, None, low[:, R:R + N], low[:, R + N:], self.rates, self.skip, xz[:, inner:], state,
-                           ctx.row_start, ctx.state_slots, y)
+                           ctx.row_start, ctx.state_slots, y, in_order=act == F32)
         if accumulate_into is None:
             return self.out(y, out_dtype=F32)
         self.out(y, residual=accumulate_into)

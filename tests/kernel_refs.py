@@ -468,7 +468,7 @@ def rows_times_table(a, table, ids, off, out):
     return out
 
 
-def selective_scan(x, dt, dt_bias, B, C, A, D, z, state, row_start, slots, out):
+def selective_scan(x, dt, dt_bias, B, C, A, D, z, state, row_start, slots, out, in_order=False):
     inner, N = A.shape
     step = torch.nn.functional.softplus(dt.double() + (dt_bias.double() if dt_bias is not None else 0.0))
     for slot, lo, hi in _requests(row_start, slots):

@@ -553,8 +553,12 @@ def test_queries_and_keys_normed_whole_and_written_to_the_cache(dtype, H, Hkv, d
 # ---- a state per channel and state index, gates on results, rows of a table, routing in groups, experts without a gate ----
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("inner,N,lengths", [(16, 16, [5]), (37, 1, [1, 9, 1]), (50, 5, [3, 1, 40]), (24, 24, [1, 1, 1, 1]), (19, 40, [33, 2]),
-                                             (8, 100, [7, 12]), (5, 256, [6]), (130, 8, [70])])
-def test_selective_scan(dtype, inner, N, lengths):
+                                             (8, 100, [7, 12]), (5, 256, [6]), (130, 8, [70]), (22, 16, [300, 1, 77]), (9, 30, [150, 64]),
+                                             (7, 50, [129]), (6, 70, [200])])
+@pytest.mark.parametrize("in_order", [False, True])
+def test_selective_scan(dtype, inner, N, lengths, in_order):
+    """Portions, single rows and padding; long portions of few requests go the way of rows shared out among waves unless
+    `in_order` (up to 64 states a channel), so both ways are held against the reference."""
     row_start, slots, T = tables(lengths, ([3, -1, 0, 2, 1] * 2)[:len(lengths)] if len(lengths) > 1 else [1])
     wide = torch.randn(T, 2 * inner + 3, device=DEV)                       # x and z as columns of wider rows
     low = torch.randn(T, 4 + 2 * N, device=DEV)
@@ -571,7 +575,7 @@ def test_selective_scan(dtype, inner, N, lengths):
         torch.random.set_rng_state(keep[0]), torch.cuda.set_rng_state(keep[1])
         args = make(z, d, b)
         host = [a.detach().cpu().clone() if isinstance(a, torch.Tensor) else a for a in args]
-        ops.selective_scan(*args)
+        ops.selective_scan(*args, in_order=in_order)
         ref.selective_scan(*host)
         live = [i for i, s in enumerate(slots.tolist()) if s >= 0]
         rows = torch.cat([torch.arange(row_start[i], row_start[i + 1]) for i in live])
@@ -581,7 +585,7 @@ def test_selective_scan(dtype, inner, N, lengths):
 
 
 def test_selective_scan_cut_anywhere_gives_the_same_bits():
-    inner, N, T = 21, 12, 47
+    inner, N, T = 21, 12, 147
     x, dt, z = (torch.randn(T, inner, device=DEV) for _ in range(3))
     B, C = torch.randn(T, N, device=DEV), torch.randn(T, N, device=DEV)
     A = -torch.exp(torch.rand(inner, N, device=DEV) * 3 - 2)
@@ -592,12 +596,16 @@ def test_selective_scan_cut_anywhere_gives_the_same_bits():
         state, out = torch.zeros(1, inner * N, device=DEV), torch.zeros(T, inner, device=DEV)
         for a, b in zip(cuts[:-1], cuts[1:]):
             rs = torch.tensor([0, b - a], dtype=torch.int32, device=DEV)
-            ops.selective_scan(x[a:b], dt[a:b], None, B[a:b], C[a:b], A, D, z[a:b], state, rs, one, out[a:b])
+            ops.selective_scan(x[a:b], dt[a:b], None, B[a:b], C[a:b], A, D, z[a:b], state, rs, one, out[a:b], in_order=True)
         return out, state
     whole = run([0, T])
     for cuts in ([0, 1, 2, 3, T], [0, 5, 7, 40, 41, T], list(range(T + 1))):
         got = run(cuts)
         assert torch.equal(got[0], whole[0]) and torch.equal(got[1], whole[1]), cuts
+    # the rows shared out among waves: the same to rounding
+    state, out = torch.zeros(1, inner * N, device=DEV), torch.zeros(T, inner, device=DEV)
+    ops.selective_scan(x, dt, None, B, C, A, D, z, state, torch.tensor([0, T], dtype=torch.int32, device=DEV), one, out)
+    close(out, whole[0]), close(state, whole[1])
 
 
 @pytest.mark.parametrize("dtype", DT)
