@@ -35,7 +35,7 @@ extern "C" int dn_gemm(const void* A, int lda, const void* W, const float* bias,
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (lda < K && !(packed & PACKED_A))) return DN_ERR_SHAPE;
   if ((packed & PACKED_W) && K % 8 != 0) return DN_ERR_SHAPE;      // (the plain kernels take any K)
-  if (epilogue < EPI_NONE || epilogue > EPI_GELU_ERF) return DN_ERR_SHAPE;
+  if (epilogue < EPI_NONE || epilogue > EPI_RELU2) return DN_ERR_SHAPE;
   if (resid != nullptr && epilogue != EPI_NONE) return DN_ERR_SHAPE;
   if ((packed & (PACKED_A | PACKED_C)) && (!(packed & PACKED_W) || M > 256)) return DN_ERR_SHAPE;
   if ((packed & PACKED_C) && (resid != nullptr || out_dtype != DN_BF16 || N % 32 != 0)) return DN_ERR_SHAPE;
@@ -169,7 +169,7 @@ extern "C" int dn_gemm_norm_in(const void* A, int lda, const float* stats, const
   if (M < 1 || M > 64 || N < 1 || K < 16 || K % 16 != 0 || K > 4096 || (lda != 0 && lda < K) || !stats || !c1 || !c2 || !C)
     return DN_ERR_SHAPE;
   if (M <= 16 ? lda == 0 : (K < 1024 || K > 2048)) return DN_ERR_SHAPE;
-  if (epilogue < EPI_NONE || epilogue > EPI_GELU_ERF) return DN_ERR_SHAPE;
+  if (epilogue < EPI_NONE || epilogue > EPI_RELU2) return DN_ERR_SHAPE;
   const int packed = PACKED_W | (lda == 0 ? PACKED_A : 0);
   if (!skinny::takes(A, lda, W, M, K, packed) || reinterpret_cast<uintptr_t>(stats) % 8 != 0) return DN_ERR_SHAPE;
   KVScatter kv{};

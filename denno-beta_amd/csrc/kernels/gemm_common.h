@@ -8,6 +8,7 @@
 #define EPI_NONE 0
 #define EPI_GELU_TANH 1
 #define EPI_GELU_ERF 2
+#define EPI_RELU2 3      // max(v, 0)^2
 
 __device__ __forceinline__ float apply_epilogue(float v, int epi) {
   if (epi == EPI_GELU_TANH) {
@@ -15,6 +16,7 @@ __device__ __forceinline__ float apply_epilogue(float v, int epi) {
     return 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
   }
   if (epi == EPI_GELU_ERF) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+  if (epi == EPI_RELU2) return fmaxf(v, 0.f) * fmaxf(v, 0.f);
   return v;
 }
 
@@ -27,6 +29,7 @@ __device__ __forceinline__ float apply_epilogue_fast(float v, int epi) {
     return v * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-2.8853900817779268f * u));
   }
   if (epi == EPI_GELU_ERF) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+  if (epi == EPI_RELU2) return fmaxf(v, 0.f) * fmaxf(v, 0.f);
   return v;
 }
 

@@ -363,6 +363,83 @@ __global__ __launch_bounds__(256) void rows_times_table_kernel(const void* a, in
   }
 }
 
+// A token input in one launch, for steps of few rows (where five launches cost more than their work): with e the `dim`
+// columns from `off` of the table's row that the row's token picks, g = gelu_tanh(W_gate x) * e, y = W_proj g,
+// x += y / sqrt(mean(y^2) + eps) * weight.  One workgroup of sixteen waves a row: the stream's row goes to LDS; a wave
+// takes a column of g at a time (the row times a row of W_gate, summed over the wave), g in LDS; then a thread a column of
+// y (a row of W_proj times g), y in LDS; the squares summed wave by wave in order.  W_gate [dim, width] and W_proj
+// [width, dim] in rows, 32-bit or bfloat16; sums in 32-bit.  VEC: bfloat16 matrices whose rows are whole pieces of 16
+// bytes: a lane asks for 16 bytes at a time and for all of a column's pieces before it uses the first.
+template <bool VEC>
+__global__ __launch_bounds__(1024) void token_input_kernel(float* x, size_t ldx, const void* wg, const void* wp, int w_dt, const void* table,
+                                                           int t_dt, size_t ldt, int off, const int* ids, int n_rows, const float* weight,
+                                                           int width, int dim, float eps) {
+  extern __shared__ float lds[];      // the row [width], g [dim], y [width]
+  __shared__ float sh[16];
+  float* xs = lds;
+  float* g = lds + width;
+  float* y = g + dim;
+  float* row = x + static_cast<size_t>(blockIdx.x) * ldx;
+  const int id = ids[blockIdx.x];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int c = threadIdx.x; c < width; c += 1024) xs[c] = row[c];
+  __syncthreads();
+  for (int j = wave; j < dim; j += 16) {
+    float acc = 0.f;
+    if (VEC) {
+      const uint4* wrow = reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(wg) + static_cast<size_t>(j) * width);
+#pragma unroll 4
+      for (int p = lane; p < width / 8; p += 64) {
+        const uint4 w = wrow[p];
+        const uint32_t q[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          acc = fmaf(__uint_as_float(q[k] << 16), xs[8 * p + 2 * k], acc);
+          acc = fmaf(__uint_as_float(q[k] & 0xffff0000u), xs[8 * p + 2 * k + 1], acc);
+        }
+      }
+    } else {
+      for (int c = lane; c < width; c += 64) acc = fmaf(load_as(wg, static_cast<size_t>(j) * width + c, w_dt), xs[c], acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) {
+      const float u = 0.7978845608028654f * (acc + 0.044715f * acc * acc * acc);
+      const float e = (id >= 0 && id < n_rows) ? load_as(table, static_cast<size_t>(id) * ldt + off + j, t_dt) : __builtin_nanf("");
+      g[j] = 0.5f * acc * (1.0f + tanhf(u)) * e;
+    }
+  }
+  __syncthreads();
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < width; c += 1024) {
+    float acc = 0.f;
+    if (VEC) {
+      const uint4* wrow = reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(wp) + static_cast<size_t>(c) * dim);
+#pragma unroll 8
+      for (int p = 0; p < dim / 8; ++p) {
+        const uint4 w = wrow[p];
+        const uint32_t q[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          acc = fmaf(__uint_as_float(q[k] << 16), g[8 * p + 2 * k], acc);
+          acc = fmaf(__uint_as_float(q[k] & 0xffff0000u), g[8 * p + 2 * k + 1], acc);
+        }
+      }
+    } else {
+      for (int j = 0; j < dim; ++j) acc = fmaf(load_as(wp, static_cast<size_t>(c) * dim + j, w_dt), g[j], acc);
+    }
+    y[c] = acc;
+    ss = fmaf(acc, acc, ss);
+  }
+  ss = wave_sum(ss);
+  if (lane == 0) sh[wave] = ss;
+  __syncthreads();
+  float total = 0.f;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) total += sh[w];
+  const float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
+  for (int c = threadIdx.x; c < width; c += 1024) row[c] = fmaf(y[c] * inv, weight ? weight[c] : 1.0f, xs[c]);
+}
+
 // ---- activations of projections that feed a recurrence or a gate --------------------------------------------
 enum { ACT_SILU = 0, ACT_SIGMOID = 1, ACT_TANH = 2, ACT_EXP_NEG_EXP = 3, ACT_BOUNDED_SIGMOID = 4, ACT_EXP_NEG_SOFTPLUS = 5, ACT_XIELU = 6,
        ACT_RELU2 = 7 };
@@ -800,12 +877,15 @@ __global__ __launch_bounds__(WAVES * 64) void gate_scan_kernel(const float* a, s
 // Over each request's rows in order, per channel c and state index n:
 //   dt = log(1 + e^(dt_in[t, c] + dt_bias[c]));  S[c, n] <- exp(dt A[c, n]) S[c, n] + dt x[t, c] B[t, n]
 //   y[t, c] = sum_n S[c, n] C[t, n] + D[c] x[t, c];  out[t, c] = y * silu(z[t, c])
+// x is what a short convolution and its activation left, 32-bit or bfloat16; everything else that enters is 32-bit.
 // A channel lies on 16 neighbouring lanes; lane l of them keeps the states n = l, l + 16, ... (PER of them) in registers
 // from a portion's first row to its last, and the sum over n is joined inside the row of 16 lanes, always in one order.
 // The rows are asked for TB at a time.  The same kernel for portions and for decoded tokens; a row's result depends on
 // the state before it alone, so how a prompt is cut changes nothing.
 struct SelectiveArgs {
-  const float *x, *dt, *dt_bias, *B, *C, *A, *D, *z;
+  const void* x;      // 32-bit or bfloat16 (x_dt): what the convolution left
+  int x_dt;
+  const float *dt, *dt_bias, *B, *C, *A, *D, *z;
   size_t ldx, ldd, ldb, ldc, ldz;
   float* state;
   size_t slot_stride;
@@ -845,7 +925,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(SelectiveArgs a) {
 #pragma unroll
     for (int i = 0; i < TB; ++i) {
       const size_t t = min(t0 + i, row1 - 1);
-      fx[i] = a.x[t * a.ldx + cc], fd[i] = a.dt[t * a.ldd + cc];
+      fx[i] = load_as(a.x, t * a.ldx + cc, a.x_dt), fd[i] = a.dt[t * a.ldd + cc];
       fz[i] = a.z ? a.z[t * a.ldz + cc] : 0.f;
 #pragma unroll
       for (int j = 0; j < PER; ++j) fb[i][j] = a.B[t * a.ldb + nn[j]], fc[i][j] = a.C[t * a.ldc + nn[j]];
@@ -950,7 +1030,7 @@ __global__ __launch_bounds__(WAVES * 64) void selective_scan_runs_kernel(Selecti
   float fx, fs, fb[TB][PER], fc[TB][PER];
   auto fetch = [&](int t0) {
     const size_t t = min(t0 + min(my, TB - 1), row1 - 1);
-    fx = a.x[t * a.ldx + cc];
+    fx = load_as(a.x, t * a.ldx + cc, a.x_dt);
     fs = steps ? a.dt[t * a.ldd + cc] : (a.z ? a.z[t * a.ldz + cc] : 0.f);
 #pragma unroll
     for (int i = 0; i < TB; ++i) {
@@ -1552,14 +1632,14 @@ int dn_rows_times_table(const void* a, int a_dt, long long lda, const void* tabl
   return dn_launch_status();
 }
 
-int dn_selective_scan(const float* x, long long ldx, const float* dt, long long ldd, const float* dt_bias, const float* B, long long ldb,
+int dn_selective_scan(const void* x, int x_dt, long long ldx, const float* dt, long long ldd, const float* dt_bias, const float* B, long long ldb,
                       const float* C, long long ldc, const float* A, const float* D, const float* z, long long ldz, float* state,
                       long long slot_stride, const int* row_start, const int* slots, int S, int T, int inner, int N, void* out,
                       int out_dt, long long ldo, int in_order, hipStream_t stream) {
-  if (!float_kind(out_dt)) return DN_ERR_DTYPE;
+  if (!float_kind(out_dt) || !float_kind(x_dt)) return DN_ERR_DTYPE;
   if (inner < 1 || N < 1 || N > 256 || S > 65535 || slot_stride < static_cast<long long>(inner) * N) return DN_ERR_SHAPE;
   if (S == 0) return 0;
-  const SelectiveArgs a{x, dt, dt_bias, B, C, A, D, z, static_cast<size_t>(ldx), static_cast<size_t>(ldd), static_cast<size_t>(ldb),
+  const SelectiveArgs a{x, x_dt, dt, dt_bias, B, C, A, D, z, static_cast<size_t>(ldx), static_cast<size_t>(ldd), static_cast<size_t>(ldb),
                         static_cast<size_t>(ldc), static_cast<size_t>(ldz), state, static_cast<size_t>(slot_stride), row_start, slots,
                         inner, N, out, out_dt, static_cast<size_t>(ldo)};
   const int per = (N + 15) / 16;
@@ -1577,6 +1657,23 @@ int dn_selective_scan(const float* x, long long ldx, const float* dt, long long 
   else if (per <= 4) hipLaunchKernelGGL(selective_scan_kernel<4>, grid, dim3(256), 0, stream, a);
   else if (per <= 8) hipLaunchKernelGGL(selective_scan_kernel<8>, grid, dim3(256), 0, stream, a);
   else hipLaunchKernelGGL(selective_scan_kernel<16>, grid, dim3(256), 0, stream, a);
+  return dn_launch_status();
+}
+
+int dn_token_input(float* x, long long ldx, const void* wg, const void* wp, int w_dt, const void* table, int t_dt, long long ldt, int off,
+                   const int* ids, int n_rows, const float* weight, int T, int width, int dim, float eps, hipStream_t stream) {
+  if (!float_kind(w_dt) || !float_kind(t_dt)) return DN_ERR_DTYPE;
+  if (width < 1 || dim < 1 || off < 0 || off + dim > ldt || n_rows < 1 || (2 * static_cast<long long>(width) + dim) * 4 > 60000) return DN_ERR_SHAPE;
+  if (T == 0) return 0;
+  const size_t lds = (2 * static_cast<size_t>(width) + dim) * sizeof(float);
+  const bool vec = w_dt == DN_BF16 && width % 8 == 0 && dim % 8 == 0 && reinterpret_cast<uintptr_t>(wg) % 16 == 0 &&
+                   reinterpret_cast<uintptr_t>(wp) % 16 == 0;
+  if (vec)
+    hipLaunchKernelGGL(token_input_kernel<true>, dim3(T), dim3(1024), lds, stream, x, static_cast<size_t>(ldx), wg, wp, w_dt, table, t_dt,
+                       static_cast<size_t>(ldt), off, ids, n_rows, weight, width, dim, eps);
+  else
+    hipLaunchKernelGGL(token_input_kernel<false>, dim3(T), dim3(1024), lds, stream, x, static_cast<size_t>(ldx), wg, wp, w_dt, table, t_dt,
+                       static_cast<size_t>(ldt), off, ids, n_rows, weight, width, dim, eps);
   return dn_launch_status();
 }
 

@@ -15,7 +15,7 @@ from ..build import load_library
 
 F32, BF16 = 0, 1
 _CODE = {torch.float32: F32, torch.bfloat16: BF16}
-EPILOGUES = {"none": 0, "gelu_tanh": 1, "gelu_erf": 2}
+EPILOGUES = {"none": 0, "gelu_tanh": 1, "gelu_erf": 2, "relu2": 3}
 
 _libs = {}
 
@@ -150,8 +150,9 @@ def _declare(name, lib):
             "dn_streams_write": [P, c_longlong, I, P, P, P, c_longlong, P, c_longlong, P, P, F, P, P, F, P, I, c_longlong, I, I, P],
             "dn_norm_pair_write": [P, c_longlong, I, I, P, P, F, P, c_longlong, P, P, P, I, I, I, I, I, I, P],
             "dn_head_gate": [P, I, c_longlong, I, P, c_longlong, P, I, c_longlong, I, I, I, P],
+            "dn_token_input": [P, c_longlong, P, P, I, P, I, c_longlong, I, P, I, P, I, I, I, F, P],
             "dn_rows_times_table": [P, I, c_longlong, P, I, c_longlong, I, P, I, P, I, c_longlong, I, I, P],
-            "dn_selective_scan": [P, c_longlong, P, c_longlong, P, P, c_longlong, P, c_longlong, P, P, P, c_longlong, P, c_longlong,
+            "dn_selective_scan": [P, I, c_longlong, P, c_longlong, P, P, c_longlong, P, c_longlong, P, P, P, c_longlong, P, c_longlong,
                                   P, P, I, I, I, I, P, I, c_longlong, I, P],
         },
         "grouped": {
@@ -1321,15 +1322,38 @@ def rows_times_table(a, table, ids, off, out):
     return out
 
 
+TOKEN_INPUT_ROWS_MAX = 64      # steps of more rows make a token input from matrix products
+
+
+def token_input(x, w_gate, w_proj, table, ids, off, weight, eps):
+    """x[t, :] += y / sqrt(mean(y^2) + eps) * weight with y = w_proj (gelu_tanh(w_gate x[t, :]) * table[ids[t], off : off + dim]),
+    one launch for steps of few rows.  x: 32-bit rows, changed in place; w_gate [dim, width] and w_proj [width, dim] in rows,
+    both 32-bit or both bfloat16; weight: 32-bit [width] or None; sums in 32-bit."""
+    _dev(x, "x", (torch.float32,), 2), _dev(w_gate, "w_gate", _FLOATS, 2), _dev(w_proj, "w_proj", (w_gate.dtype,), 2)
+    _dev(table, "table", _FLOATS, 2), _dev(ids, "ids", _I32, 1)
+    T, width = x.shape
+    dim = w_gate.shape[0]
+    _need(tuple(w_gate.shape) == (dim, width) and tuple(w_proj.shape) == (width, dim) and w_gate.is_contiguous() and w_proj.is_contiguous()
+          and ids.is_contiguous() and ids.shape[0] == T and off >= 0 and off + dim <= table.shape[1], "token_input: shapes")
+    _need((2 * width + dim) * 4 <= 60000, lambda: f"token_input: a row of {width} and {dim} columns does not fit the workgroup's memory")
+    _f32vec(weight, "weight", width)
+    _ok(_lib("sequence").dn_token_input(x.data_ptr(), _rows(x, "x"), w_gate.data_ptr(), w_proj.data_ptr(), _CODE[w_gate.dtype], table.data_ptr(),
+                                        _CODE[table.dtype], _rows(table, "table"), off, ids.data_ptr(), table.shape[0], _ptr(weight), T, width,
+                                        dim, float(eps), _stream()), "token_input")
+    return x
+
+
 def selective_scan(x, dt, dt_bias, B, C, A, D, z, state, row_start, slots, out, in_order=False):
     """A state per channel c and state index n with a decay of its own, over each request's rows in order:
       step = log(1 + e^(dt[t, c] + dt_bias[c]));  S[c, n] <- exp(step * A[c, n]) S[c, n] + step * x[t, c] * B[t, n]
       y[t, c] = sum_n S[c, n] C[t, n] + D[c] x[t, c];  out[t, c] = y * silu(z[t, c])      (z None: y as it is)
-    x, dt, z: 32-bit [T, inner]; B, C: 32-bit [T, N] (all may be columns of wider rows); A: 32-bit [inner, N]; dt_bias, D:
+    x [T, inner]: 32-bit or bfloat16 (what a convolution and its activation left); dt, z: 32-bit [T, inner]; B, C: 32-bit
+    [T, N] (all may be columns of wider rows); A: 32-bit [inner, N]; dt_bias, D:
     32-bit [inner] or None; state: 32-bit [slots, inner * N], read and written at the requests' slots; out [T, inner].
     in_order: every request's rows are walked one after the other, which gives the same bits however a prompt is cut; else
     long portions of few requests are shared out among a workgroup's waves and joined, which changes a result by rounding."""
-    for t, name in ((x, "x"), (dt, "dt"), (B, "B"), (C, "C")) + (((z, "z"),) if z is not None else ()):
+    _dev(x, "x", _FLOATS, 2)
+    for t, name in ((dt, "dt"), (B, "B"), (C, "C")) + (((z, "z"),) if z is not None else ()):
         _dev(t, name, (torch.float32,), 2)
     _dev(out, "out", _FLOATS, 2), _dev(A, "A", (torch.float32,), 2)
     T, inner = x.shape
@@ -1340,7 +1364,7 @@ def selective_scan(x, dt, dt_bias, B, C, A, D, z, state, row_start, slots, out, 
     _need(1 <= N <= 256, lambda: f"selective_scan: {N} states a channel; the kernel keeps up to 256 on a channel's lanes")
     _f32vec(dt_bias, "dt_bias", inner), _f32vec(D, "D", inner)
     stride = _history(state, inner * N, "selective_scan")
-    _ok(_lib("sequence").dn_selective_scan(x.data_ptr(), _rows(x, "x"), dt.data_ptr(), _rows(dt, "dt"), _ptr(dt_bias), B.data_ptr(),
+    _ok(_lib("sequence").dn_selective_scan(x.data_ptr(), _CODE[x.dtype], _rows(x, "x"), dt.data_ptr(), _rows(dt, "dt"), _ptr(dt_bias), B.data_ptr(),
                                            _rows(B, "B"), C.data_ptr(), _rows(C, "C"), A.data_ptr(), _ptr(D), _ptr(z),
                                            _rows(z, "z") if z is not None else 0, state.data_ptr(), stride, row_start.data_ptr(),
                                            slots.data_ptr(), S, T, inner, N, out.data_ptr(), _CODE[out.dtype], _rows(out, "out"),

@@ -247,6 +247,11 @@ class RoutedExperts(Part):
         ops.moe_combine(out, None if on_input else wts, accumulate_into)
         if self.shared:
             n = self.shared["inner"]
+            if not self.gated and not self.token_gate:
+                # max(W_up h, 0)^2 in the first product's epilogue, the second product added where the experts' results are
+                f = self.shared_up(h, out_dtype=self.shared_down.weight.dtype, epilogue="relu2")
+                self.shared_down(f, residual=accumulate_into)
+                return accumulate_into if returns else None
             gu = self.shared_up(h, out_dtype=torch.float32)
             f = torch.empty((T, n), dtype=self.shared_down.weight.dtype, device=dev)
             if self.gated:

@@ -387,8 +387,8 @@ class Mamba1(Part):
     B: N | C: N]; the step of a channel is dt_c = log(1 + e^(W_dt dt + bias)_c); A = -e^(A_log), [inner, N].  Per channel c and
     state index n: S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n; y_c = sum_n S[c, n] C_n + D_c x_c; y times silu(z);
     then the output projection.  State: S in 32-bit and the convolution's last taps - 1 inputs.  32-bit are the
-    projections' results that enter the recurrence (x behind its convolution, dt, B, C, z), the steps, the decays, the
-    state and its sums; the products' operands are the engine's."""
+    projections' results that enter the recurrence (dt, B, C, z; the convolution reads its input in 32-bit), the steps, the
+    decays, the state and its sums; the products' operands, and x behind its convolution and silu, are the engine's."""
     graph_safe = True
     returns_rows = True
     libraries = ("sequence",)
@@ -434,7 +434,8 @@ class Mamba1(Part):
         inner, N, R = self.inner, self.state_dim, self.dt_rank
         state, past = cache.state[:, :inner * N], cache.state[:, inner * N:]
         xz = self.proj(h, out_dtype=F32)
-        x = torch.empty((T, inner), dtype=F32, device=dev)
+        # (what the convolution and its silu leave is in the engine's precision: the next product's rows as they are)
+        x = torch.empty((T, inner), dtype=act, device=dev)
         ops.conv_rows(xz, self.conv, past, ctx.row_start, ctx.state_slots, x, identity=False, act="silu", bias=self.conv_bias)
         if self.taps > 1 and cache.writes:
             ops.history_update(xz[:, :inner], past, ctx.row_start, ctx.state_slots)

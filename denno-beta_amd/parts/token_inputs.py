@@ -16,7 +16,8 @@ F32 = torch.float32
 @TOKEN_INPUTS.register("gated_table_rows")
 class GatedTableRows(Part):
     """e = table[token, offset : offset + dim];  g = act(W_gate x) * e;  y = W_proj g;  x += y / sqrt(mean(y^2) + eps) * w,
-    with x the stream's rows as they stand (not normed).  act: "gelu_tanh"."""
+    with x the stream's rows as they stand (not normed).  act: "gelu_tanh".  Steps of many rows run it as two products with
+    the activation in the first one's epilogue; steps of up to `ops.TOKEN_INPUT_ROWS_MAX` rows as one kernel."""
     graph_safe = True
     libraries = ("sequence",)
 
@@ -39,6 +40,10 @@ class GatedTableRows(Part):
         super().bind(tensors, runtime)
         self.gate.bind(tensors), self.proj.bind(tensors)
         self.norm = tensors[self.norm_name]
+        # the matrices in rows as well, for the kernel that makes a step of few rows in one launch
+        wg, wp = tensors[self.gate.weight_name], tensors[self.proj.weight_name]
+        fits = (2 * self.width + self.dim) * 4 <= 60000 and wg.dtype == wp.dtype
+        self.gate_rows, self.proj_rows = (wg.contiguous(), wp.contiguous()) if runtime.act_dtype != F32 and fits else (None, None)
         rows = runtime.tables.get(self.table)
         if rows is None:
             raise KeyError(f"gated_table_rows: the model has no table {self.table!r}")
@@ -48,6 +53,9 @@ class GatedTableRows(Part):
 
     def forward(self, x, ctx):
         act = self.runtime.act_dtype
+        if self.gate_rows is not None and x.shape[0] <= ops.TOKEN_INPUT_ROWS_MAX:
+            # a step of few rows: one launch (the bfloat16 engine; the 32-bit engine keeps the products' one order of sums)
+            return ops.token_input(x, self.gate_rows, self.proj_rows, self.rows, ctx.tokens, self.offset, self.norm, self.eps)
         g = self.gate(x, out_dtype=act, epilogue=self.activation)
         ops.rows_times_table(g, self.rows, ctx.tokens, self.offset, g)
         ops.rmsnorm_add(self.proj(g, out_dtype=F32), self.norm, None, 1.0, self.eps, x)

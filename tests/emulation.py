@@ -9,7 +9,7 @@ from denno_beta_amd.kernels import ops
 
 _NAMES = ["embed", "embed_sum", "logits_post", "layernorm", "kv_write", "cast", "linear", "linear_qkv", "linear_norm_out", "linear_norm_in", "attention", "sample", "sample_top", "sample_full", "penalties", "history_append",
           "rmsnorm", "rmsnorm_add", "depth_mix", "unit_heads", "concat_cast", "conv_rows", "conv_heads", "rotary_runs", "history_update", "shift_mix", "rotary", "activate", "gated", "state_scan",
-          "head_norm", "step_sizes", "gate_scan", "streams_read", "streams_write", "norm_pair_write", "pair_rows", "heads_linear", "head_gate", "rows_times_table", "selective_scan", "moe_route", "moe_plan", "moe_up", "moe_down", "moe_combine"]
+          "head_norm", "step_sizes", "gate_scan", "streams_read", "streams_write", "norm_pair_write", "pair_rows", "heads_linear", "head_gate", "rows_times_table", "token_input", "selective_scan", "moe_route", "moe_plan", "moe_up", "moe_down", "moe_combine"]
 
 
 @contextlib.contextmanager

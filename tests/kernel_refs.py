@@ -82,6 +82,8 @@ def linear(a, w, bias=None, out=None, epilogue="none", residual=None):
         y = torch.nn.functional.gelu(y, approximate="tanh")
     elif epilogue == "gelu_erf":
         y = torch.nn.functional.gelu(y)
+    elif epilogue == "relu2":
+        y = torch.relu(y) ** 2
     elif epilogue != "none":
         raise ValueError(epilogue)
     out.copy_(y)
@@ -117,6 +119,8 @@ def linear_norm_in(copy, stats, c1, c2, eps, w, out, epilogue="none", kv=None, n
         y = torch.nn.functional.gelu(y, approximate="tanh")
     elif epilogue == "gelu_erf":
         y = torch.nn.functional.gelu(y)
+    elif epilogue == "relu2":
+        y = torch.relu(y) ** 2
     if kv is None:
         out.copy_(y)
         return out
@@ -466,6 +470,16 @@ def rows_times_table(a, table, ids, off, out):
     n = a.shape[1]
     out.copy_(a.float() * table[ids.long(), off:off + n].float())
     return out
+
+
+def token_input(x, w_gate, w_proj, table, ids, off, weight, eps):
+    dim = w_gate.shape[0]
+    z = x @ w_gate.float().T
+    g = torch.nn.functional.gelu(z, approximate="tanh") * table[ids.long(), off:off + dim].float()
+    y = g @ w_proj.float().T
+    n = y / torch.sqrt((y * y).mean(dim=-1, keepdim=True) + eps)
+    x += n if weight is None else n * weight
+    return x
 
 
 def selective_scan(x, dt, dt_bias, B, C, A, D, z, state, row_start, slots, out, in_order=False):

@@ -699,3 +699,42 @@ def test_experts_without_a_gate(dtype, T, E, top, ff, width):
         close(y2, hy, dtype, "moe_up, packed")
     z = torch.randn(T, ff, device=DEV)
     close(ops.activate(z, "relu2", torch.zeros(T, ff, dtype=dtype, device=DEV)), torch.relu(z) ** 2, dtype)
+
+
+@pytest.mark.parametrize("wdt", DT)
+@pytest.mark.parametrize("T,width,dim", [(1, 24, 1), (8, 100, 5), (64, 1024, 64), (3, 36, 16), (5, 2048, 250), (2, 4096, 256), (7, 40, 8)])
+def test_a_token_input_in_one_launch(wdt, T, width, dim):
+    x = torch.randn(T, width + 3, device=DEV)[:, :width] * 2
+    wg = (torch.randn(dim, width, device=DEV) / width ** 0.5).to(wdt)
+    wp = (torch.randn(width, dim, device=DEV) / dim ** 0.5).to(wdt)
+    table = torch.randn(31, 3 * dim + 2, device=DEV).to(wdt)
+    ids = torch.randint(0, 31, (T,), dtype=torch.int32, device=DEV)
+    w = torch.randn(width, device=DEV)
+    for weight, off in ((w, 0), (None, 2 * dim + 2)):
+        mine, host = x.clone(), x.cpu().clone()
+        ops.token_input(mine, wg, wp, table, ids, off, weight, 1e-5)
+        ref.token_input(host, wg.cpu(), wp.cpu(), table.cpu(), ids.cpu(), off, None if weight is None else weight.cpu(), 1e-5)
+        close(mine, host, torch.float32, "token_input")
+
+
+def test_selective_scan_reads_rounded_channels():
+    inner, N = 20, 16
+    row_start, slots, T = tables([90, 3], [1, 0])
+    x = torch.randn(T, inner, device=DEV).to(torch.bfloat16)
+    dt, z = torch.randn(T, inner, device=DEV), torch.randn(T, inner, device=DEV)
+    B, C = torch.randn(T, N, device=DEV), torch.randn(T, N, device=DEV)
+    A = -torch.exp(torch.rand(inner, N, device=DEV) * 3 - 2)
+    for in_order in (True, False):
+        both("selective_scan", lambda: (x, dt, None, B, C, A, None, z, torch.zeros(2, inner * N, device=DEV), row_start, slots,
+                                        torch.zeros(T, inner, device=DEV), in_order), [8, 11])
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("M,N,K", [(3, 40, 24), (70, 96, 64), (300, 128, 160)])
+def test_a_product_that_ends_in_a_squared_relu(dtype, M, N, K):
+    a = torch.randn(M, K, device=DEV).to(dtype)
+    w = (torch.randn(N, K, device=DEV) / K ** 0.5).to(dtype)
+    want = ref.linear(a.cpu(), w.cpu(), None, torch.zeros(M, N, dtype=dtype), epilogue="relu2")
+    close(ops.linear(a, w, None, torch.zeros(M, N, dtype=dtype, device=DEV), epilogue="relu2"), want, dtype, "rows")
+    if dtype == torch.bfloat16:
+        close(ops.linear(a, ops.pack_matrix(w), None, torch.zeros(M, N, dtype=dtype, device=DEV), epilogue="relu2"), want, dtype, "packed")
