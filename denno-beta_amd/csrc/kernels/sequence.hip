@@ -384,28 +384,45 @@ __global__ __launch_bounds__(1024) void token_input_kernel(float* x, size_t ldx,
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   for (int c = threadIdx.x; c < width; c += 1024) xs[c] = row[c];
   __syncthreads();
-  for (int j = wave; j < dim; j += 16) {
-    float acc = 0.f;
+  // (a wave takes four columns of g at a time, j0 + 16 m, and asks for a piece of each of their rows before it uses the first)
+  for (int j0 = wave; j0 < dim; j0 += 64) {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
     if (VEC) {
-      const uint4* wrow = reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(wg) + static_cast<size_t>(j) * width);
-#pragma unroll 4
-      for (int p = lane; p < width / 8; p += 64) {
-        const uint4 w = wrow[p];
-        const uint32_t q[4] = {w.x, w.y, w.z, w.w};
+      const uint4* wrow[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          acc = fmaf(__uint_as_float(q[k] << 16), xs[8 * p + 2 * k], acc);
-          acc = fmaf(__uint_as_float(q[k] & 0xffff0000u), xs[8 * p + 2 * k + 1], acc);
+      for (int m = 0; m < 4; ++m)
+        wrow[m] = reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(wg) + static_cast<size_t>(min(j0 + 16 * m, dim - 1)) * width);
+#pragma unroll 2
+      for (int p = lane; p < width / 8; p += 64) {
+        uint4 w[4];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) w[m] = wrow[m][p];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          const uint32_t q[4] = {w[m].x, w[m].y, w[m].z, w[m].w};
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            acc[m] = fmaf(__uint_as_float(q[k] << 16), xs[8 * p + 2 * k], acc[m]);
+            acc[m] = fmaf(__uint_as_float(q[k] & 0xffff0000u), xs[8 * p + 2 * k + 1], acc[m]);
+          }
         }
       }
     } else {
-      for (int c = lane; c < width; c += 64) acc = fmaf(load_as(wg, static_cast<size_t>(j) * width + c, w_dt), xs[c], acc);
+      for (int c = lane; c < width; c += 64) {
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+          acc[m] = fmaf(load_as(wg, static_cast<size_t>(min(j0 + 16 * m, dim - 1)) * width + c, w_dt), xs[c], acc[m]);
+      }
     }
-    acc = wave_sum(acc);
-    if (lane == 0) {
-      const float u = 0.7978845608028654f * (acc + 0.044715f * acc * acc * acc);
-      const float e = (id >= 0 && id < n_rows) ? load_as(table, static_cast<size_t>(id) * ldt + off + j, t_dt) : __builtin_nanf("");
-      g[j] = 0.5f * acc * (1.0f + tanhf(u)) * e;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const int j = j0 + 16 * m;
+      const float v = wave_sum(acc[m]);
+      if (lane == 0 && j < dim) {
+        const float u = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+        const float e = (id >= 0 && id < n_rows) ? load_as(table, static_cast<size_t>(id) * ldt + off + j, t_dt) : __builtin_nanf("");
+        g[j] = 0.5f * v * (1.0f + tanhf(u)) * e;
+      }
     }
   }
   __syncthreads();

@@ -272,6 +272,8 @@ ALONE = {
     "attention_not_turned": [with_mlp(attention(3, 3, 16, 8, dims=None, window=11), None)],
     "latent": [with_mlp(latent(2, 8, 4, 8, 8, window=0), None)],
     "latent_window_stretched": [with_mlp(latent(3, 6, 6, 10, 5, window=6, scaled=scaling(3.0, 8, 2.0, 1.0)), None)],
+    # a latent too wide for one key of the attention kernels: every head's own keys and values are kept instead
+    "latent_kept_by_heads": [with_mlp(latent(2, 8, 4, 12, 262, window=9), None)],
     "dense": [with_mlp(scan(8, 2, 1, 2), dense(28))],
     "experts": [with_mlp(scan(8, 2, 1, 2), moe(12, 6, 3, None, 1.0, None))],
     "experts_in_groups": [with_mlp(scan(8, 2, 1, 2), moe(12, 8, 2, (4, 2), 2.0, None))],
