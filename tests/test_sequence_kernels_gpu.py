@@ -553,13 +553,15 @@ def test_queries_and_keys_normed_whole_and_written_to_the_cache(dtype, H, Hkv, d
 # ---- a state per channel and state index, gates on results, rows of a table, routing in groups, experts without a gate ----
 @pytest.mark.parametrize("dtype", DT)
 @pytest.mark.parametrize("inner,N,lengths", [(16, 16, [5]), (37, 1, [1, 9, 1]), (50, 5, [3, 1, 40]), (24, 24, [1, 1, 1, 1]), (19, 40, [33, 2]),
-                                             (8, 100, [7, 12]), (5, 256, [6]), (130, 8, [70]), (22, 16, [300, 1, 77]), (9, 30, [150, 64]),
+                                             (8, 100, [7, 12]), (5, 256, [6]), (130, 8, [70]), (22, 16, [300, 1, 77]), (9, 30, [150, 64]), (2100, 16, [1] * 20), (1100, 20, [1, 2, 1] * 11),
                                              (7, 50, [129]), (6, 70, [200])])
 @pytest.mark.parametrize("in_order", [False, True])
 def test_selective_scan(dtype, inner, N, lengths, in_order):
     """Portions, single rows and padding; long portions of few requests go the way of rows shared out among waves unless
     `in_order` (up to 64 states a channel), so both ways are held against the reference."""
-    row_start, slots, T = tables(lengths, ([3, -1, 0, 2, 1] * 2)[:len(lengths)] if len(lengths) > 1 else [1])
+    n_slots = max(5, len(lengths))
+    slot_of = [3, -1, 0, 2, 1] if len(lengths) <= 5 else [(-1 if i % 7 == 1 else i) for i in range(len(lengths))]
+    row_start, slots, T = tables(lengths, slot_of[:len(lengths)] if len(lengths) > 1 else [1])
     wide = torch.randn(T, 2 * inner + 3, device=DEV)                       # x and z as columns of wider rows
     low = torch.randn(T, 4 + 2 * N, device=DEV)
     dt = torch.randn(T, inner, device=DEV) * 2 - 1
@@ -567,7 +569,7 @@ def test_selective_scan(dtype, inner, N, lengths, in_order):
     D, bias = torch.randn(inner, device=DEV), torch.randn(inner, device=DEV)
 
     def make(z, d, b):
-        state = torch.randn(5, inner * N + 7, device=DEV)[:, :inner * N]
+        state = torch.randn(n_slots, inner * N + 7, device=DEV)[:, :inner * N]
         return (wide[:, :inner], dt, b, low[:, 4:4 + N], low[:, 4 + N:], A, d, z, state, row_start, slots,
                 torch.zeros(T, inner, dtype=dtype, device=DEV))
     keep = torch.random.get_rng_state(), torch.cuda.get_rng_state()
