@@ -62,10 +62,12 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const void* x, int x_dt, s
 
 // x[t, :] += mult * (y[t, :] / sqrt(mean(y^2) + eps) * weight) * scale: the norm of a sublayer's result, added into the
 // stream (scale: a vector, or none).  gate: y is y * sigmoid(gate[t, :]) first, under the norm's sums too (a gate on the
-// sublayer's result).  One workgroup a row, the sums as in rmsnorm_kernel.
+// sublayer's result).  next_out: the row as it then stands, normed for whoever reads the stream next (next_w, next_eps): a
+// launch less between two sublayers.  One workgroup a row, the sums as in rmsnorm_kernel.
 __global__ __launch_bounds__(256) void rmsnorm_add_kernel(const void* y, int y_dt, size_t ldy, const float* weight, const float* scale,
                                                           float mult, float* x, size_t ldx, int width, float eps, const float* gate,
-                                                          size_t ldg) {
+                                                          size_t ldg, const float* next_w, float next_eps, void* next_out, int next_dt,
+                                                          size_t ldn) {
   __shared__ float sh[4];
   const size_t src = static_cast<size_t>(blockIdx.x) * ldy, dst = static_cast<size_t>(blockIdx.x) * ldx;
   const float* g = gate ? gate + static_cast<size_t>(blockIdx.x) * ldg : nullptr;
@@ -77,13 +79,24 @@ __global__ __launch_bounds__(256) void rmsnorm_add_kernel(const void* y, int y_d
   }
   ss = block_sum_256(ss, sh);
   const float inv = 1.0f / sqrtf(ss / static_cast<float>(width) + eps);
+  float after = 0.f;
   for (int c = threadIdx.x; c < width; c += 256) {
     float v = load_as(y, src + c, y_dt);
     if (g) v *= 1.0f / (1.0f + expf(-g[c]));
     v *= inv;
     if (weight) v *= weight[c];
     if (scale) v *= scale[c];
-    x[dst + c] = fmaf(mult, v, x[dst + c]);
+    const float sum = fmaf(mult, v, x[dst + c]);
+    x[dst + c] = sum;
+    after = fmaf(sum, sum, after);
+  }
+  if (!next_out) return;
+  // the norm that reads the stream next, on the row as it stands now: the sums as rmsnorm_kernel makes them (the same bits)
+  after = block_sum_256(after, sh);
+  const float inv2 = 1.0f / sqrtf(after / static_cast<float>(width) + next_eps);
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const float v = x[dst + c] * inv2;      // (the thread's own store)
+    store_as(next_out, static_cast<size_t>(blockIdx.x) * ldn + c, next_dt, next_w ? v * next_w[c] : v);
   }
 }
 
@@ -373,7 +386,8 @@ __global__ __launch_bounds__(256) void rows_times_table_kernel(const void* a, in
 template <bool VEC>
 __global__ __launch_bounds__(1024) void token_input_kernel(float* x, size_t ldx, const void* wg, const void* wp, int w_dt, const void* table,
                                                            int t_dt, size_t ldt, int off, const int* ids, int n_rows, const float* weight,
-                                                           int width, int dim, float eps) {
+                                                           int width, int dim, float eps, const float* next_w, float next_eps,
+                                                           void* next_out, int next_dt, size_t ldn) {
   extern __shared__ float lds[];      // the row [width], g [dim], y [width]
   __shared__ float sh[16];
   float* xs = lds;
@@ -454,7 +468,25 @@ __global__ __launch_bounds__(1024) void token_input_kernel(float* x, size_t ldx,
 #pragma unroll
   for (int w = 0; w < 16; ++w) total += sh[w];
   const float inv = 1.0f / sqrtf(total / static_cast<float>(width) + eps);
-  for (int c = threadIdx.x; c < width; c += 1024) row[c] = fmaf(y[c] * inv, weight ? weight[c] : 1.0f, xs[c]);
+  float after = 0.f;
+  for (int c = threadIdx.x; c < width; c += 1024) {
+    const float sum = fmaf(y[c] * inv, weight ? weight[c] : 1.0f, xs[c]);
+    row[c] = sum;
+    y[c] = sum;      // (the thread's own place)
+    after = fmaf(sum, sum, after);
+  }
+  if (!next_out) return;
+  // the norm that reads the stream next, on the row as it stands now
+  after = wave_sum(after);
+  __syncthreads();
+  if (lane == 0) sh[wave] = after;
+  __syncthreads();
+  total = 0.f;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) total += sh[w];
+  const float inv2 = 1.0f / sqrtf(total / static_cast<float>(width) + next_eps);
+  for (int c = threadIdx.x; c < width; c += 1024)
+    store_as(next_out, static_cast<size_t>(blockIdx.x) * ldn + c, next_dt, next_w ? y[c] * inv2 * next_w[c] : y[c] * inv2);
 }
 
 // ---- activations of projections that feed a recurrence or a gate --------------------------------------------
@@ -1362,12 +1394,14 @@ int dn_rmsnorm(const void* x, int x_dt, long long ldx, const float* weight, void
 }
 
 int dn_rmsnorm_add(const void* y, int y_dt, long long ldy, const float* weight, const float* scale, float mult, float* x, long long ldx,
-                   int T, int width, float eps, const float* gate, long long ldg, hipStream_t stream) {
-  if (!float_kind(y_dt)) return DN_ERR_DTYPE;
-  if (T < 0 || width < 1 || (gate && ldg < width)) return DN_ERR_SHAPE;
+                   int T, int width, float eps, const float* gate, long long ldg, const float* next_w, float next_eps, void* next_out,
+                   int next_dt, long long ldn, hipStream_t stream) {
+  if (!float_kind(y_dt) || (next_out && !float_kind(next_dt))) return DN_ERR_DTYPE;
+  if (T < 0 || width < 1 || (gate && ldg < width) || (next_out && ldn < width)) return DN_ERR_SHAPE;
   if (T == 0) return 0;
   hipLaunchKernelGGL(rmsnorm_add_kernel, dim3(T), dim3(256), 0, stream, y, y_dt, static_cast<size_t>(ldy), weight, scale, mult, x,
-                     static_cast<size_t>(ldx), width, eps, gate, static_cast<size_t>(ldg));
+                     static_cast<size_t>(ldx), width, eps, gate, static_cast<size_t>(ldg), next_w, next_eps, next_out, next_dt,
+                     static_cast<size_t>(ldn));
   return dn_launch_status();
 }
 
@@ -1701,8 +1735,9 @@ int dn_selective_scan(const void* x, int x_dt, long long ldx, const float* dt, l
 }
 
 int dn_token_input(float* x, long long ldx, const void* wg, const void* wp, int w_dt, const void* table, int t_dt, long long ldt, int off,
-                   const int* ids, int n_rows, const float* weight, int T, int width, int dim, float eps, hipStream_t stream) {
-  if (!float_kind(w_dt) || !float_kind(t_dt)) return DN_ERR_DTYPE;
+                   const int* ids, int n_rows, const float* weight, int T, int width, int dim, float eps, const float* next_w,
+                   float next_eps, void* next_out, int next_dt, long long ldn, hipStream_t stream) {
+  if (!float_kind(w_dt) || !float_kind(t_dt) || (next_out && (!float_kind(next_dt) || ldn < width))) return DN_ERR_DTYPE;
   if (width < 1 || dim < 1 || off < 0 || off + dim > ldt || n_rows < 1 || (2 * static_cast<long long>(width) + dim) * 4 > 60000) return DN_ERR_SHAPE;
   if (T == 0) return 0;
   const size_t lds = (2 * static_cast<size_t>(width) + dim) * sizeof(float);
@@ -1710,10 +1745,12 @@ int dn_token_input(float* x, long long ldx, const void* wg, const void* wp, int 
                    reinterpret_cast<uintptr_t>(wp) % 16 == 0;
   if (vec)
     hipLaunchKernelGGL(token_input_kernel<true>, dim3(T), dim3(1024), lds, stream, x, static_cast<size_t>(ldx), wg, wp, w_dt, table, t_dt,
-                       static_cast<size_t>(ldt), off, ids, n_rows, weight, width, dim, eps);
+                       static_cast<size_t>(ldt), off, ids, n_rows, weight, width, dim, eps, next_w, next_eps, next_out, next_dt,
+                       static_cast<size_t>(ldn));
   else
     hipLaunchKernelGGL(token_input_kernel<false>, dim3(T), dim3(1024), lds, stream, x, static_cast<size_t>(ldx), wg, wp, w_dt, table, t_dt,
-                       static_cast<size_t>(ldt), off, ids, n_rows, weight, width, dim, eps);
+                       static_cast<size_t>(ldt), off, ids, n_rows, weight, width, dim, eps, next_w, next_eps, next_out, next_dt,
+                       static_cast<size_t>(ldn));
   return dn_launch_status();
 }
 

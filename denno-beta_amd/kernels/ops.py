@@ -130,7 +130,7 @@ def _declare(name, lib):
         "sequence": {
             "dn_rmsnorm": [P, I, c_longlong, P, P, I, c_longlong, P, I, I, F, P],
             "dn_concat_cast": [P, c_longlong, I, P, c_longlong, I, P, I, I, P],
-            "dn_rmsnorm_add": [P, I, c_longlong, P, P, F, P, c_longlong, I, I, F, P, c_longlong, P],
+            "dn_rmsnorm_add": [P, I, c_longlong, P, P, F, P, c_longlong, I, I, F, P, c_longlong, P, F, P, I, c_longlong, P],
             "dn_depth_mix": [P, c_longlong, I, P, P, c_longlong, P],
             "dn_unit_heads": [P, c_longlong, P, c_longlong, I, I, I, F, F, P],
             "dn_conv_rows": [P, c_longlong, P, P, P, P, P, I, I, I, I, I, I, P, I, c_longlong, c_longlong, P],
@@ -150,7 +150,7 @@ def _declare(name, lib):
             "dn_streams_write": [P, c_longlong, I, P, P, P, c_longlong, P, c_longlong, P, P, F, P, P, F, P, I, c_longlong, I, I, P],
             "dn_norm_pair_write": [P, c_longlong, I, I, P, P, F, P, c_longlong, P, P, P, I, I, I, I, I, I, P],
             "dn_head_gate": [P, I, c_longlong, I, P, c_longlong, P, I, c_longlong, I, I, I, P],
-            "dn_token_input": [P, c_longlong, P, P, I, P, I, c_longlong, I, P, I, P, I, I, I, F, P],
+            "dn_token_input": [P, c_longlong, P, P, I, P, I, c_longlong, I, P, I, P, I, I, I, F, P, F, P, I, c_longlong, P],
             "dn_rows_times_table": [P, I, c_longlong, P, I, c_longlong, I, P, I, P, I, c_longlong, I, I, P],
             "dn_selective_scan": [P, I, c_longlong, P, c_longlong, P, P, c_longlong, P, c_longlong, P, P, P, c_longlong, P, c_longlong,
                                   P, P, I, I, I, I, P, I, c_longlong, I, P],
@@ -1005,10 +1005,21 @@ def rmsnorm(x, weight, eps, out, rows=None):
     return out
 
 
-def rmsnorm_add(y, weight, scale, mult, eps, x, gate=None):
+def _then(then, T, width, what):
+    """then = (weight or None, eps, out): the norm that reads the stream next, made by the same kernel -> its five arguments."""
+    if then is None:
+        return 0, 0.0, 0, 0, 0
+    w, eps, out = then
+    _f32vec(w, "next weight", width), _dev(out, "next out", _FLOATS, 2)
+    _need(tuple(out.shape) == (T, width), lambda: f"{what}: the next norm's rows")
+    return _ptr(w), float(eps), out.data_ptr(), _CODE[out.dtype], _rows(out, "next out")
+
+
+def rmsnorm_add(y, weight, scale, mult, eps, x, gate=None, then=None):
     """x[t, :] += mult * (y[t, :] / sqrt(mean(y[t, :]^2) + eps) * weight) * scale; weight and scale: 32-bit vectors or None;
     x: 32-bit rows (the stream), changed in place; statistics in 32-bit.  gate: 32-bit [T, width] (columns of wider rows):
-    y is y * sigmoid(gate) first, under the norm too."""
+    y is y * sigmoid(gate) first, under the norm too.  then = (weight or None, eps, out): out[t, :] = x[t, :] / sqrt(mean(x[t, :]^2)
+    + eps) * weight on the rows as they then stand, the same bits as `rmsnorm` behind this call."""
     _dev(y, "y", _FLOATS, 2), _dev(x, "x", (torch.float32,), 2)
     T, width = y.shape
     _need(tuple(x.shape) == (T, width), "rmsnorm_add: shapes")
@@ -1018,7 +1029,8 @@ def rmsnorm_add(y, weight, scale, mult, eps, x, gate=None):
         _need(tuple(gate.shape) == (T, width), "rmsnorm_add: gate")
     _ok(_lib("sequence").dn_rmsnorm_add(y.data_ptr(), _CODE[y.dtype], _rows(y, "y"), _ptr(weight), _ptr(scale), float(mult),
                                         x.data_ptr(), _rows(x, "x"), T, width, float(eps), _ptr(gate),
-                                        _rows(gate, "gate") if gate is not None else 0, _stream()), "rmsnorm_add")
+                                        _rows(gate, "gate") if gate is not None else 0, *_then(then, T, width, "rmsnorm_add"),
+                                        _stream()), "rmsnorm_add")
     return x
 
 
@@ -1325,10 +1337,11 @@ def rows_times_table(a, table, ids, off, out):
 TOKEN_INPUT_ROWS_MAX = 64      # steps of more rows make a token input from matrix products
 
 
-def token_input(x, w_gate, w_proj, table, ids, off, weight, eps):
+def token_input(x, w_gate, w_proj, table, ids, off, weight, eps, then=None):
     """x[t, :] += y / sqrt(mean(y^2) + eps) * weight with y = w_proj (gelu_tanh(w_gate x[t, :]) * table[ids[t], off : off + dim]),
     one launch for steps of few rows.  x: 32-bit rows, changed in place; w_gate [dim, width] and w_proj [width, dim] in rows,
-    both 32-bit or both bfloat16; weight: 32-bit [width] or None; sums in 32-bit."""
+    both 32-bit or both bfloat16; weight: 32-bit [width] or None; sums in 32-bit.  then: as in `rmsnorm_add`: the norm that reads
+    the stream next, in the same launch."""
     _dev(x, "x", (torch.float32,), 2), _dev(w_gate, "w_gate", _FLOATS, 2), _dev(w_proj, "w_proj", (w_gate.dtype,), 2)
     _dev(table, "table", _FLOATS, 2), _dev(ids, "ids", _I32, 1)
     T, width = x.shape
@@ -1339,7 +1352,7 @@ def token_input(x, w_gate, w_proj, table, ids, off, weight, eps):
     _f32vec(weight, "weight", width)
     _ok(_lib("sequence").dn_token_input(x.data_ptr(), _rows(x, "x"), w_gate.data_ptr(), w_proj.data_ptr(), _CODE[w_gate.dtype], table.data_ptr(),
                                         _CODE[table.dtype], _rows(table, "table"), off, ids.data_ptr(), table.shape[0], _ptr(weight), T, width,
-                                        dim, float(eps), _stream()), "token_input")
+                                        dim, float(eps), *_then(then, T, width, "token_input"), _stream()), "token_input")
     return x
 
 

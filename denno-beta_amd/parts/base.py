@@ -83,6 +83,9 @@ class Runtime:
     # next reads it first (set by the model), and the rows that the block before has read for this one in its last write's kernel
     next_read: Optional[tuple] = None
     stream_rows: Optional[torch.Tensor] = None
+    # rows that the kernel which last changed the stream has normed already for the norm that reads it next: (norm, rows), or
+    # None; whoever changes the stream otherwise clears it (the model does at a step's start and end)
+    normed_rows: Optional[tuple] = None
     # the model's further tables by name (DecoderSpec.tables), for parts that pick rows of them (set by the model)
     tables: Dict[str, torch.Tensor] = field(default_factory=dict)
 

@@ -204,15 +204,31 @@ class GatedSandwichBlock(SandwichBlock):
         return ([self.norm1, self.mixer, self.gate1, self.post1]
                 + ([self.norm2, self.ffn, self.gate2, self.post2] if self.has_ffn else []) + ([self.side] if self.has_side else []))
 
+    def first_norm(self):
+        """The norm that reads the residual stream first in this block."""
+        return self.norm1
+
     def forward(self, x, ctx, caches, runtime):
+        # The norm in front of a sublayer is made by the kernel that takes the sublayer before into the stream (the norm
+        # behind it, or the token input), where that norm is a plain one: a launch less per sublayer; across blocks the rows
+        # travel in runtime.normed_rows with the norm they were made for.
+        act = runtime.act_dtype
         runtime.stream_stats = None
-        h = self.norm1.forward(x, runtime.act_dtype)
-        self.post1.add_into(self._result(self.mixer, x, h, ctx, caches[0]), x, gate=self.gate1.logits(h))
+        came, runtime.normed_rows = runtime.normed_rows, None
+        h = came[1] if came is not None and came[0] is self.norm1 else self.norm1.forward(x, act)
+        nxt = runtime.next_norm
+        y = self._result(self.mixer, x, h, ctx, caches[0])
+        then = self.norm2 if self.has_ffn else (None if self.has_side else nxt)
+        h = self.post1.add_into(y, x, gate=self.gate1.logits(h), then=then, out_dtype=act)
         if self.has_ffn:
-            h = self.norm2.forward(x, runtime.act_dtype)
-            self.post2.add_into(self._result(self.ffn, x, h, ctx), x, gate=self.gate2.logits(h))
+            if h is None:
+                h = self.norm2.forward(x, act)
+            y = self._result(self.ffn, x, h, ctx)
+            h = self.post2.add_into(y, x, gate=self.gate2.logits(h), then=None if self.has_side else nxt, out_dtype=act)
         if self.has_side:
-            self.side.forward(x, ctx)
+            h = self.side.forward(x, ctx, then=nxt)
+        if h is not None and nxt is not None:
+            runtime.normed_rows = (nxt, h)
 
 
 @ARRANGEMENTS.register("multi_stream")

@@ -290,7 +290,7 @@ class DecoderModel:
                     picked = getattr(ctx, t.index)
                 parts.append((self.extra_tables[t.name], picked, t.scale))
             ops.embed_sum(parts, x)
-        rt.stream_stats = rt.stream_deferred = None      # nobody has left anything for a norm of these rows yet
+        rt.stream_stats = rt.stream_deferred = rt.normed_rows = None      # nobody has left anything for a norm of these rows yet
         if self.embedding_norm is not None:
             x = self.embedding_norm.forward(x, torch.float32)
         x0 = x.clone() if self.injections else None      # (the blocks add into x in place)
@@ -310,7 +310,7 @@ class DecoderModel:
             if call.inject is not None:
                 if rt.stream_deferred is not None:
                     rt.stream_deferred.flush(x)
-                rt.stream_stats = rt.stream_deferred = None
+                rt.stream_stats = rt.stream_deferred = rt.normed_rows = None
                 both = ops.concat_cast(x, x0, torch.empty((ctx.T, 2 * self.spec.width), dtype=rt.act_dtype, device=rt.device))
                 x = self.injections[call.inject](both, out_dtype=torch.float32)
             nxt = self.blocks[order[i + 1].layer] if i + 1 < len(order) else None
@@ -324,14 +324,14 @@ class DecoderModel:
             if kept is not None:
                 if rt.stream_deferred is not None:
                     rt.stream_deferred.flush(x)
-                rt.stream_stats = rt.stream_deferred = None
+                rt.stream_stats = rt.stream_deferred = rt.normed_rows = None
                 if x.data_ptr() != kept[i + 1].data_ptr():      # (an injection made new rows)
                     kept[i + 1].copy_(x)
                 w = self.averages.get(i)
                 x = ops.depth_mix(kept, i + 2, w, kept[i + 2]) if w is not None else ops.depth_mix(kept[i + 1:], 1, self._one, kept[i + 2])
         if rt.stream_deferred is not None:
             rt.stream_deferred.flush(x)
-        rt.stream_stats = rt.next_norm = rt.stream_deferred = None
+        rt.stream_stats = rt.next_norm = rt.stream_deferred = rt.normed_rows = None
         rt.next_takes_deferred = False
         if ctx.R == 0:
             return torch.empty((0, self.spec.vocab), dtype=torch.float32, device=rt.device)

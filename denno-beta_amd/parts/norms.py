@@ -97,5 +97,17 @@ class StreamRMSNorm(RMSNorm):
         super().bind(tensors, runtime)
         self.scale = tensors[self.scale_name] if self.scale_name else None
 
-    def add_into(self, y, x, gate=None):
-        return ops.rmsnorm_add(y, self.weight, self.scale, self.mult, self.eps, x, gate=gate)
+    def add_into(self, y, x, gate=None, then=None, out_dtype=None):
+        """then: the norm that reads the stream next; if it is a plain `rmsnorm`, its rows come out of the same kernel and
+        are returned (else None, and that norm runs as a kernel of its own)."""
+        nxt = following_norm(then, x, out_dtype)
+        ops.rmsnorm_add(y, self.weight, self.scale, self.mult, self.eps, x, gate=gate, then=nxt)
+        return nxt[2] if nxt is not None else None
+
+
+def following_norm(norm, x, out_dtype):
+    """(weight, eps, rows to fill) for a kernel that, having changed the stream's rows x, norms them for `norm` as well; None
+    where `norm` is none or not a plain root-mean-square norm over the whole row."""
+    if norm is None or type(norm) is not RMSNorm or norm.width != x.shape[1] or out_dtype is None:
+        return None
+    return norm.weight, norm.eps, torch.empty(x.shape, dtype=out_dtype, device=x.device)

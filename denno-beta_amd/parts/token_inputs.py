@@ -51,14 +51,20 @@ class GatedTableRows(Part):
             raise ValueError(f"gated_table_rows: columns {self.offset} .. {self.offset + self.dim} of a table with {rows.shape[1]}")
         self.rows = rows
 
-    def forward(self, x, ctx):
+    def forward(self, x, ctx, then=None):
+        """then: the norm that reads the stream next: where it is a plain `rmsnorm` its rows come out of the last kernel and
+        are returned (else None)."""
+        from .norms import following_norm
         act = self.runtime.act_dtype
+        nxt = following_norm(then, x, act)
         if self.gate_rows is not None and x.shape[0] <= ops.TOKEN_INPUT_ROWS_MAX:
             # a step of few rows: one launch (the bfloat16 engine; the 32-bit engine keeps the products' one order of sums)
-            return ops.token_input(x, self.gate_rows, self.proj_rows, self.rows, ctx.tokens, self.offset, self.norm, self.eps)
-        g = self.gate(x, out_dtype=act, epilogue=self.activation)
-        ops.rows_times_table(g, self.rows, ctx.tokens, self.offset, g)
-        ops.rmsnorm_add(self.proj(g, out_dtype=F32), self.norm, None, 1.0, self.eps, x)
+            ops.token_input(x, self.gate_rows, self.proj_rows, self.rows, ctx.tokens, self.offset, self.norm, self.eps, then=nxt)
+        else:
+            g = self.gate(x, out_dtype=act, epilogue=self.activation)
+            ops.rows_times_table(g, self.rows, ctx.tokens, self.offset, g)
+            ops.rmsnorm_add(self.proj(g, out_dtype=F32), self.norm, None, 1.0, self.eps, x, then=nxt)
+        return nxt[2] if nxt is not None else None
 
 
 @TOKEN_INPUTS.register("none")
@@ -69,5 +75,5 @@ class NoTokenInput(Part):
     def __init__(self):
         pass
 
-    def forward(self, x, ctx):
+    def forward(self, x, ctx, then=None):
         return None

@@ -266,7 +266,14 @@ def rmsnorm(x, weight, eps, out, rows=None):
     return out
 
 
-def rmsnorm_add(y, weight, scale, mult, eps, x, gate=None):
+def _then(then, x):
+    if then is not None:
+        w, eps, out = then
+        n = x / torch.sqrt((x * x).mean(dim=-1, keepdim=True) + eps)
+        out.copy_(n if w is None else n * w)
+
+
+def rmsnorm_add(y, weight, scale, mult, eps, x, gate=None, then=None):
     src = y.float()
     if gate is not None:
         src = src * torch.sigmoid(gate.float())
@@ -276,6 +283,7 @@ def rmsnorm_add(y, weight, scale, mult, eps, x, gate=None):
     if scale is not None:
         n = n * scale
     x += mult * n
+    _then(then, x)
     return x
 
 
@@ -472,13 +480,14 @@ def rows_times_table(a, table, ids, off, out):
     return out
 
 
-def token_input(x, w_gate, w_proj, table, ids, off, weight, eps):
+def token_input(x, w_gate, w_proj, table, ids, off, weight, eps, then=None):
     dim = w_gate.shape[0]
     z = x @ w_gate.float().T
     g = torch.nn.functional.gelu(z, approximate="tanh") * table[ids.long(), off:off + dim].float()
     y = g @ w_proj.float().T
     n = y / torch.sqrt((y * y).mean(dim=-1, keepdim=True) + eps)
     x += n if weight is None else n * weight
+    _then(then, x)
     return x
 
 

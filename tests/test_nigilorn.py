@@ -115,11 +115,11 @@ def folders(tmp_path_factory):
     return get
 
 
-def runner_for(folder, dtype, device, cache_tokens, max_live=4, page_size=16):
+def runner_for(folder, dtype, device, cache_tokens, max_live=4, page_size=16, graphs=True):
     from denno_beta_amd.config import EngineOptions
     from denno_beta_amd.engine import ModelRunner
     return ModelRunner.from_folder(folder, EngineOptions(dtype=dtype, device=device, page_size=page_size,
-                                                         cache_tokens=cache_tokens, max_live=max_live))
+                                                         cache_tokens=cache_tokens, max_live=max_live, use_graphs=graphs))
 
 
 _plain = {}
@@ -395,6 +395,44 @@ def test_the_stream_after_every_layer(backend, folders):
     for i, want in enumerate(streams):
         d = (seen[i].double() - want).abs().max() / want.abs().max()
         assert d < 2e-5, f"the stream behind layer {i} differs by {d:.3g} of its largest entry"
+
+
+def test_norms_in_front_of_sublayers_come_out_of_the_kernels_before(backend, folders):
+    """The norm in front of a sublayer is made by the kernel that takes the sublayer before it into the stream: a whole step
+    launches the norm's own kernel for the first layer and for the head only, and the logits are those of the norms as
+    kernels of their own (on the GPU the same bits)."""
+    from denno_beta_amd.kernels import ops
+    from denno_beta_amd.parts import norms, token_inputs
+    cfg = CONFIGS["P"][0]
+    folder = folders("P", "float32")
+    seqs = seqs_for(cfg, [21, 70], seed=15)
+    steps = U.whole_trace(seqs) + [dict(s, step=10 + i) for i, s in enumerate(U.tail_decode_trace([seqs[0]], 5))]
+    for i, s in enumerate(steps[2:]):
+        s["entries"][0]["id"], s["end"] = "again", (["again"] if s["end"] else [])
+    for dtype in ("float32", "bfloat16"):
+        calls = []
+        real, real_following = ops.rmsnorm, norms.following_norm
+
+        def spy(x, weight, eps, out, rows=None):
+            if out.shape[1] == cfg["width"]:
+                calls.append(out.shape[0])
+            return real(x, weight, eps, out, rows)
+        ops.rmsnorm = spy
+        try:
+            fused = U.replay(runner_for(folder, dtype, backend, 256, graphs=False), steps)      # (every step kernel by kernel)
+            per_step = len(calls) / len(steps)
+            norms.following_norm = lambda norm, x, out_dtype: None
+            apart = U.replay(runner_for(folder, dtype, backend, 256), steps)
+        finally:
+            ops.rmsnorm, norms.following_norm = real, real_following
+        assert per_step == 2, f"{per_step} norm kernels a step; the first layer's and the head's are two"
+        for rid in fused:
+            if backend == "cpu":
+                assert_rows(fused[rid], apart[rid], "float32", f"{dtype} {rid}", 1e-5 if dtype == "float32" else 0.02)
+            elif dtype == "float32":
+                assert torch.equal(fused[rid], apart[rid]), f"{rid}: the norm inside the kernel before gives other bits"
+            else:       # (the token input of few rows sums a row over sixteen waves, the norm's own kernel over four)
+                assert_rows(fused[rid], apart[rid], "float32", f"{dtype} {rid}", 0.02)
 
 
 # ----------------------------------------------------------------------------------------------------------------

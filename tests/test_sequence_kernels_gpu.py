@@ -622,6 +622,15 @@ def test_norm_of_a_gated_result_added_into_the_stream(width, dtype):
     ops.rmsnorm_add(y, w, None, 1.0, 1e-5, x, gate=gate)
     ref.rmsnorm_add(y.cpu(), w.cpu(), None, 1.0, 1e-5, hx, gate=gate.cpu())
     close(x, hx)
+    # with the norm that reads the stream next in the same launch: the same bits as that norm's own kernel behind it
+    w2 = torch.randn(width, device=DEV)
+    for nw in (w2, None):
+        x1, x2 = x.clone(), x.clone()
+        out = torch.zeros(T, width + 2, dtype=dtype, device=DEV)[:, :width]
+        ops.rmsnorm_add(y, w, None, 0.5, 1e-5, x1, gate=gate, then=(nw, 1e-6, out))
+        ops.rmsnorm_add(y, w, None, 0.5, 1e-5, x2, gate=gate)
+        assert torch.equal(x1, x2)
+        assert torch.equal(out, ops.rmsnorm(x2, nw, 1e-6, torch.zeros(T, width, dtype=dtype, device=DEV)))
 
 
 @pytest.mark.parametrize("dtype", DT)
@@ -717,6 +726,10 @@ def test_a_token_input_in_one_launch(wdt, T, width, dim):
         ops.token_input(mine, wg, wp, table, ids, off, weight, 1e-5)
         ref.token_input(host, wg.cpu(), wp.cpu(), table.cpu(), ids.cpu(), off, None if weight is None else weight.cpu(), 1e-5)
         close(mine, host, torch.float32, "token_input")
+        again, nxt = x.clone(), torch.zeros(T, width, dtype=wdt, device=DEV)
+        ops.token_input(again, wg, wp, table, ids, off, weight, 1e-5, then=(weight, 1e-6, nxt))
+        assert torch.equal(again, mine)
+        close(nxt, ref.rmsnorm(mine.cpu(), None if weight is None else weight.cpu(), 1e-6, torch.zeros(T, width)), wdt, "token_input, the next norm")
 
 
 def test_selective_scan_reads_rounded_channels():
